@@ -1,0 +1,138 @@
+/*
+ * ladder_hip.h -- C ABI of libladder_hip.so: the gfx950 (MI355X) kernels behind the per-rank
+ * forward pass of the Ladder-Residual transformer.
+ *
+ * The reference (mayank31398/ladder-residual-inference) has no FFI: its boundary is the Python
+ * module API of gpt_fast/.  Every entry point below therefore replaces a call site of a
+ * PyTorch / Triton / third-party kernel in the reference, cited per function as file:line under
+ * the reference root.  The host side (the gpt_fast package shipped beside the HIP sources) binds
+ * them with ctypes and keeps the reference's module names and signatures.
+ *
+ * Conventions, all entry points:
+ *   - every tensor argument is a DEVICE pointer to bf16 (uint16 storage) unless stated otherwise,
+ *     dense row-major, 16-byte aligned; row strides ("ld*") are in elements and multiples of 8;
+ *   - `stream` is a hipStream_t; work is only enqueued on it.  No entry point allocates,
+ *     synchronises, or touches host memory after it returns, so every call can be recorded into
+ *     a hipGraph by stream capture;
+ *   - positions are read on the DEVICE from `pos` (int32), never from the host, so a captured
+ *     decode step can be replayed after the position buffer has been advanced on the device;
+ *   - the return value is LR_OK or a negative LR_E_* code; on error nothing was launched;
+ *   - arithmetic: bf16 storage, fp32 accumulation, one round-to-nearest-even at each point where
+ *     the eager reference materialises a bf16 tensor.
+ */
+#ifndef LADDER_HIP_H
+#define LADDER_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* lr_stream_t; /* hipStream_t */
+
+enum {
+  LR_OK = 0,
+  LR_E_NULL = -1,        /* a required pointer is NULL                                   */
+  LR_E_ALIGN = -2,       /* a pointer is not 16-byte aligned or a stride is not % 8      */
+  LR_E_SHAPE = -3,       /* a size is non-positive or inconsistent                        */
+  LR_E_UNSUPPORTED = -4, /* a size the kernels are not built for (e.g. head_dim)          */
+  LR_E_LAUNCH = -5       /* the HIP runtime refused the launch                            */
+};
+
+/* Library version (major*10000 + minor*100 + patch) and text for an LR_E_* code. */
+int lr_version(void);
+const char* lr_error_string(int code);
+
+/* out[t, :] = table[idx[t], :]   -- tok_embeddings(idx), gpt_ladder_TP.py:256.
+ * idx: int64 (idx_is_i64 != 0) or int32, n_tokens entries; ids outside [0, vocab) give a zero row. */
+int lr_embed(const void* table, const void* idx, int idx_is_i64, void* out, int64_t n_tokens, int dim, int vocab,
+             lr_stream_t stream);
+
+/* out = bf16(a + bf16(b / b_div))  over n elements.  b_div == 1 is the plain add of
+ * add_tensor_forward_triton_kernel (gpt_ladder_TP.py:364-377, call sites :326-332, :346-349) and
+ * of the dense / parallel residual adds (gpt_dense_TP.py:281-282, gpt_parallel_TP.py:224);
+ * b_div == tp is desync's pre-scaled residual (gpt_desync_TP.py:369-382). `out` may alias a or b. */
+int lr_add(const void* a, const void* b, float b_div, void* out, int64_t n, lr_stream_t stream);
+
+/* Fused residual update + RMSNorm over `rows` rows of `dim`:
+ *     r = resid_in;  if (d1) r = bf16(r + d1);  if (d2) r = bf16(r + d2);
+ *     if (resid_out) resid_out = r;
+ *     normed_out = bf16( bf16( r * rsqrt(mean(r^2) + eps) ) * gain )
+ * Replaces the ladder add followed by attention_norm / ffn_norm (gpt_ladder_TP.py:326-337,
+ * :346-354), the closing x + prev_attn + prev_mlp and final norm (:280-282), and RMSNorm itself
+ * (utils.py:68-74).  d1, d2, resid_out may be NULL; resid_out may alias resid_in.  dim <= 16384. */
+int lr_add_rmsnorm(const void* resid_in, const void* d1, const void* d2, const void* gain, void* resid_out,
+                   void* normed_out, int rows, int dim, float eps, lr_stream_t stream);
+
+/* y[m, n] = bf16( sum_k x[m, k] * w[n, k] )   x [M, K] (row stride ldx), w [N, K] dense,
+ * y [M, N] (row stride ldy).  nn.Linear without bias: wqkv / wo (utils.py:191, 258), w1 / w2
+ * (utils.py:146, 148), wqkv1 (utils.py:311), output (gpt_ladder_TP.py:283).
+ * M <= 8 runs the weight-streaming GEMV, larger M the LDS-tiled MFMA GEMM.  K % 8 == 0.
+ * act_swiglu != 0: x is taken to be [M, 2K] = [u | g] (row stride ldx) and the kernel consumes
+ * bf16( bf16(silu(g)) * u ) in its place -- w2(silu(g) * u), utils.py:147-148. */
+int lr_linear(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K, int act_swiglu,
+              lr_stream_t stream);
+
+/* out[r, i] = bf16( bf16(silu(h[r, I + i])) * h[r, i] ),  h [rows, 2I] = [u | g] (row stride ldh).
+ * F.silu(g) * u after chunk(2), utils.py:147-148 and :386. */
+int lr_swiglu(const void* h, int64_t ldh, void* out, int rows, int I, lr_stream_t stream);
+
+/* RoPE on q and k plus the KV-cache write, for B*S rows of a fused projection output.
+ *   qkv [B*S, ldqkv]: columns [0, Hq*hd) = q, then Hkv*hd of k, then Hkv*hd of v (utils.py:191).
+ *   table [block_size, hd/2, 2] bf16 (cos, sin) (utils.py:103-117); pos int32 [S] on the device.
+ *   table_is_gathered == 0: the row used for token s is table[pos[s]] (the whole freqs_cis table);
+ *   table_is_gathered != 0: the caller already gathered freqs_cis[input_pos] (gpt_ladder_TP.py:255),
+ *   `table` has S rows (block_size = S) and token s uses row s.
+ * q is rotated IN PLACE; rotated k and raw v go to k_cache / v_cache [Bmax, Hkv, Smax, hd] at
+ * slot pos[s] (apply_rotary_emb utils.py:120-132, 197-198; KVCache.update utils.py:50-59,
+ * 248-250).  Rotation is done in fp32 on interleaved pairs with separately rounded products.
+ * Rows whose position is outside [0, Smax) (or outside the table) are left untouched. */
+int lr_rope_kv_write(void* qkv, int64_t ldqkv, const void* table, int table_is_gathered, const int32_t* pos,
+                     void* k_cache, void* v_cache, int B, int S, int Hq, int Hkv, int hd, int Smax, int block_size,
+                     lr_stream_t stream);
+
+/* Bytes of fp32 scratch lr_attn_decode needs for (B, Hq, hd, Smax). */
+size_t lr_attn_decode_scratch_bytes(int B, int Hq, int hd, int Smax);
+
+/* One-query attention over the contiguous KV cache (decode, S == 1):
+ *   y[b, h*hd : (h+1)*hd] = softmax_j<=pos( q[b,h] . K[b, h/G, j] / sqrt(hd) ) V[b, h/G, j]
+ * q [B, Hq*hd] (row stride ldq, already rotated), caches [Bmax, Hkv, Smax, hd], pos int32 [1] on
+ * the device, y [B, Hq*hd] (row stride ldy).  Only slots 0..pos are read; the reference reads
+ * the whole cache under a mask (repeat_interleave + F.scaled_dot_product_attention,
+ * utils.py:252-255, mask gpt_ladder_TP.py:254), which is the same function.  fp32 throughout,
+ * one rounding of y.  scratch: lr_attn_decode_scratch_bytes(). */
+int lr_attn_decode(const void* q, int64_t ldq, const void* k_cache, const void* v_cache, const int32_t* pos, void* y,
+                   int64_t ldy, int B, int Hq, int Hkv, int hd, int Smax, void* scratch, size_t scratch_bytes,
+                   lr_stream_t stream);
+
+/* Causal attention of S query tokens per sequence against the cache (prefill, S > 1):
+ * query s of row b sits at position pos[s] and sees cache slots j <= pos[s].
+ * q [B*S, Hq*hd] (row stride ldq), y [B*S, Hq*hd] (row stride ldy); the caches must already hold
+ * this call's keys (lr_rope_kv_write).  Same maths and call sites as lr_attn_decode. */
+int lr_attn_prefill(const void* q, int64_t ldq, const void* k_cache, const void* v_cache, const int32_t* pos, void* y,
+                    int64_t ldy, int B, int S, int Hq, int Hkv, int hd, int Smax, lr_stream_t stream);
+
+/* out[b] = argmax_v logits[b, v], lowest index on ties; logits [B, V] bf16 (row stride ldl),
+ * out int32 [B].  Greedy stand-in for sample() (benchmark.py:73-77): torch.argmax(logits[:, -1]). */
+int lr_argmax(const void* logits, int64_t ldl, int32_t* out, int B, int V, lr_stream_t stream);
+
+/* Device-side bookkeeping between two decode steps, what generate_using_cuda_graphs does on the
+ * host between replays (benchmark.py:208-217):
+ *     if (history) history[b, pos[0] - pos0] = next_token[b]     (slots outside [0, hist_len) skipped)
+ *     cur_token[b] = next_token[b]  for b < B;   pos[0] += 1
+ * cur_token / next_token / pos / history may be NULL to skip their part.  history int32
+ * [B, ld_hist].  Recorded after a decode step, it makes a captured step self-advancing. */
+int lr_advance(int32_t* cur_token, const int32_t* next_token, int32_t* pos, int B, int32_t* history, int64_t ld_hist,
+               int hist_len, int pos0, lr_stream_t stream);
+
+/* Tuning hook, no counterpart in the reference: force the GEMV launch configuration
+ * (rows-per-wave * 100 + K-split * 10 + unroll; 0 restores the built-in shape heuristic).
+ * Results do not depend on it beyond fp32 summation order. */
+void lr_gemv_set_cfg(int cfg);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LADDER_HIP_H */

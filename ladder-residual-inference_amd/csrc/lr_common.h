@@ -1,0 +1,73 @@
+// Shared device helpers for the gfx950 kernels: bf16 <-> fp32, 128-bit loads, wave64 reductions,
+// argument checks.  bf16 is carried as raw 16-bit words; conversions to bf16 round to nearest even
+// (v_cvt_pk_bf16_f32 on gfx950).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/ladder_hip.h"
+
+#define LR_WAVE 64
+
+typedef uint16_t u16;
+typedef uint32_t u32;
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float bf_lo(u32 p) { return __uint_as_float(p << 16); }
+__device__ __forceinline__ float bf_hi(u32 p) { return __uint_as_float(p & 0xffff0000u); }
+__device__ __forceinline__ float bf_to_f(u16 v) { return __uint_as_float(((u32)v) << 16); }
+__device__ __forceinline__ u16 f_to_bf(float f) {
+  __bf16 b = (__bf16)f;
+  return __builtin_bit_cast(u16, b);
+}
+__device__ __forceinline__ u32 pack_bf2(float lo, float hi) { return (u32)f_to_bf(lo) | ((u32)f_to_bf(hi) << 16); }
+// round an fp32 value to bf16 and back: the value a bf16 tensor would hold
+__device__ __forceinline__ float round_bf(float f) { return bf_to_f(f_to_bf(f)); }
+
+__device__ __forceinline__ uint4 ld16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ void st16(void* p, uint4 v) { *reinterpret_cast<uint4*>(p) = v; }
+
+// 8 bf16 packed in a uint4 -> 8 floats
+__device__ __forceinline__ void unpack8(const uint4& v, float* f) {
+  f[0] = bf_lo(v.x); f[1] = bf_hi(v.x); f[2] = bf_lo(v.y); f[3] = bf_hi(v.y);
+  f[4] = bf_lo(v.z); f[5] = bf_hi(v.z); f[6] = bf_lo(v.w); f[7] = bf_hi(v.w);
+}
+__device__ __forceinline__ uint4 pack8(const float* f) {
+  uint4 v;
+  v.x = pack_bf2(f[0], f[1]); v.y = pack_bf2(f[2], f[3]); v.z = pack_bf2(f[4], f[5]); v.w = pack_bf2(f[6], f[7]);
+  return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, LR_WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, LR_WAVE));
+  return v;
+}
+
+// silu in fp32 the way the eager reference evaluates it: x / (1 + exp(-x)), rounded to bf16, then
+// multiplied by u and rounded again.
+__device__ __forceinline__ float swiglu_bf(float u, float g) {
+  float s = round_bf(g / (1.0f + expf(-g)));
+  return round_bf(s * u);
+}
+
+static inline bool lr_misaligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
+
+#define LR_REQUIRE_PTR(p) \
+  do {                    \
+    if ((p) == nullptr) return LR_E_NULL; \
+    if (lr_misaligned(p)) return LR_E_ALIGN; \
+  } while (0)
+#define LR_OPTIONAL_PTR(p) \
+  do {                     \
+    if ((p) != nullptr && lr_misaligned(p)) return LR_E_ALIGN; \
+  } while (0)
+
+static inline int lr_launch_status() { return hipGetLastError() == hipSuccess ? LR_OK : LR_E_LAUNCH; }

@@ -1,0 +1,195 @@
+"""ctypes binding of libladder_hip.so (declared in include/ladder_hip.h).
+
+There is no fallback: if the shared library is missing or a call returns an error code the
+caller gets an exception.  Tensors are passed as raw device pointers plus sizes; the stream is
+torch's current HIP stream, so calls made under torch.cuda.graph() are captured."""
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_void_p
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libladder_hip.so")
+_lib = None
+
+# name -> (restype, argtypes); mirrors include/ladder_hip.h
+_PROTOS = {
+    "lr_version": (c_int, []),
+    "lr_error_string": (c_char_p, [c_int]),
+    "lr_embed": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_void_p]),
+    "lr_add": (c_int, [c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p]),
+    "lr_add_rmsnorm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float,
+                               c_void_p]),
+    "lr_linear": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
+    "lr_swiglu": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_int, c_void_p]),
+    "lr_rope_kv_write": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                 c_int, c_int, c_int, c_int, c_void_p]),
+    "lr_attn_decode_scratch_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "lr_attn_decode": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int,
+                               c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "lr_attn_prefill": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,
+                                c_int, c_int, c_int, c_int, c_void_p]),
+    "lr_argmax": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_int, c_void_p]),
+    "lr_advance": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_void_p]),
+    "lr_gemv_set_cfg": (None, [c_int]),
+}
+
+
+class LadderHipError(RuntimeError):
+    pass
+
+
+def lib_path() -> str:
+    return _LIB_PATH
+
+
+def load():
+    """Load the shared library once.  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise LadderHipError(
+                f"{_LIB_PATH} is missing: build it with `python {os.path.dirname(os.path.dirname(_LIB_PATH))}/build.py` "
+                "(hipcc, gfx950).  This package has no CPU or PyTorch fallback.")
+        lib = ctypes.CDLL(_LIB_PATH)
+        for name, (res, args) in _PROTOS.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def exported_names():
+    return list(_PROTOS)
+
+
+def _check(code: int, what: str):
+    if code != 0:
+        raise LadderHipError(f"{what} failed: {load().lr_error_string(code).decode()} ({code})")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t: torch.Tensor, dtype=torch.bfloat16) -> int:
+    assert t.is_cuda, "libladder_hip works on device tensors only"
+    assert t.dtype == dtype, f"expected {dtype}, got {t.dtype}"
+    return t.data_ptr()
+
+
+def _rows_ld(t: torch.Tensor):
+    """View a tensor as [rows, cols] with unit column stride; returns (rows, cols, row stride)."""
+    assert t.stride(-1) == 1
+    cols = t.shape[-1]
+    if t.dim() == 1:
+        return 1, cols, cols
+    rows = t.numel() // cols
+    ld = t.stride(-2)
+    # every leading dimension must be a multiple walk of the row stride
+    exp = ld
+    for d in range(t.dim() - 2, -1, -1):
+        assert t.shape[d] == 1 or t.stride(d) == exp, "tensor is not a regular [rows, cols] matrix"
+        exp *= t.shape[d]
+    return rows, cols, ld
+
+
+# ------------------------------------------------------------------------------------------------
+# thin typed wrappers
+# ------------------------------------------------------------------------------------------------
+
+def embed(table: torch.Tensor, idx: torch.Tensor, out: torch.Tensor):
+    assert idx.dtype in (torch.int64, torch.int32) and idx.is_contiguous() and idx.is_cuda
+    vocab, dim = table.shape
+    _check(load().lr_embed(_dev(table), idx.data_ptr(), int(idx.dtype == torch.int64), _dev(out), idx.numel(), dim,
+                           vocab, _stream()), "lr_embed")
+    return out
+
+
+def add(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor, b_div: float = 1.0):
+    assert a.is_contiguous() and b.is_contiguous() and out.is_contiguous() and a.numel() == b.numel() == out.numel()
+    _check(load().lr_add(_dev(a), _dev(b), float(b_div), _dev(out), a.numel(), _stream()), "lr_add")
+    return out
+
+
+def add_rmsnorm(resid_in, d1, d2, gain, resid_out, normed_out, eps: float):
+    dim = resid_in.shape[-1]
+    rows = resid_in.numel() // dim
+    for t in (resid_in, d1, d2, resid_out, normed_out):
+        assert t is None or (t.is_contiguous() and t.numel() == rows * dim)
+    assert gain.numel() == dim
+    p = lambda t: None if t is None else _dev(t)
+    _check(load().lr_add_rmsnorm(_dev(resid_in), p(d1), p(d2), _dev(gain), p(resid_out), _dev(normed_out), rows, dim,
+                                 float(eps), _stream()), "lr_add_rmsnorm")
+    return normed_out
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, act_swiglu: bool = False):
+    """out[M, N] = x[M, K] @ w[N, K]^T (x = [u | g] of width 2K when act_swiglu)."""
+    M, xc, ldx = _rows_ld(x)
+    N, K = w.shape
+    assert w.is_contiguous() and xc == (2 * K if act_swiglu else K), (x.shape, w.shape, act_swiglu)
+    Mo, No, ldy = _rows_ld(out)
+    assert (Mo, No) == (M, N), (out.shape, M, N)
+    _check(load().lr_linear(_dev(x), ldx, _dev(w), _dev(out), ldy, M, N, K, int(act_swiglu), _stream()), "lr_linear")
+    return out
+
+
+def swiglu(h: torch.Tensor, out: torch.Tensor):
+    rows, two_i, ldh = _rows_ld(h)
+    assert out.is_contiguous() and out.numel() == rows * (two_i // 2)
+    _check(load().lr_swiglu(_dev(h), ldh, _dev(out), rows, two_i // 2, _stream()), "lr_swiglu")
+    return out
+
+
+def rope_kv_write(qkv, table, table_is_gathered, pos, k_cache, v_cache, B, S, Hq, Hkv, hd):
+    rows, cols, ld = _rows_ld(qkv)
+    assert rows == B * S and pos.dtype == torch.int32 and pos.is_cuda and pos.numel() == S
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape == v_cache.shape
+    Bmax, hkv_c, Smax, hd_c = k_cache.shape
+    assert B <= Bmax and hkv_c == Hkv and hd_c == hd and table.is_contiguous() and table.shape[-2:] == (hd // 2, 2)
+    _check(load().lr_rope_kv_write(_dev(qkv), ld, _dev(table), int(bool(table_is_gathered)), pos.data_ptr(),
+                                   _dev(k_cache), _dev(v_cache), B, S, Hq, Hkv, hd, Smax, table.shape[0], _stream()),
+           "lr_rope_kv_write")
+
+
+def attn_decode_scratch_bytes(B, Hq, hd, Smax) -> int:
+    return int(load().lr_attn_decode_scratch_bytes(B, Hq, hd, Smax))
+
+
+def attn_decode(q, k_cache, v_cache, pos, y, scratch, B, Hq, Hkv, hd):
+    _, _, ldq = _rows_ld(q)
+    _, _, ldy = _rows_ld(y)
+    Smax = k_cache.shape[2]
+    assert pos.dtype == torch.int32 and pos.numel() == 1 and scratch.dtype == torch.float32
+    _check(load().lr_attn_decode(_dev(q), ldq, _dev(k_cache), _dev(v_cache), pos.data_ptr(), _dev(y), ldy, B, Hq, Hkv,
+                                 hd, Smax, scratch.data_ptr(), scratch.numel() * 4, _stream()), "lr_attn_decode")
+    return y
+
+
+def attn_prefill(q, k_cache, v_cache, pos, y, B, S, Hq, Hkv, hd):
+    _, _, ldq = _rows_ld(q)
+    _, _, ldy = _rows_ld(y)
+    Smax = k_cache.shape[2]
+    assert pos.dtype == torch.int32 and pos.numel() == S
+    _check(load().lr_attn_prefill(_dev(q), ldq, _dev(k_cache), _dev(v_cache), pos.data_ptr(), _dev(y), ldy, B, S, Hq,
+                                  Hkv, hd, Smax, _stream()), "lr_attn_prefill")
+    return y
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor):
+    B, V, ld = _rows_ld(logits)
+    assert out.dtype == torch.int32 and out.numel() == B and out.is_cuda
+    _check(load().lr_argmax(_dev(logits), ld, out.data_ptr(), B, V, _stream()), "lr_argmax")
+    return out
+
+
+def advance(cur_token, next_token, pos, B, history=None, pos0=0):
+    """cur_token <- next_token, history[:, pos - pos0] <- next_token, pos += 1, all on the device."""
+    p = lambda t: None if t is None else t.data_ptr()
+    for t in (cur_token, next_token, pos, history):
+        assert t is None or (t.dtype == torch.int32 and t.is_cuda)
+    ld, n = (history.stride(0), history.shape[1]) if history is not None else (0, 0)
+    _check(load().lr_advance(p(cur_token), p(next_token), p(pos), B, p(history), ld, n, int(pos0), _stream()),
+           "lr_advance")

@@ -1,0 +1,171 @@
+"""Model skeleton shared by GPTLadder / GPTDense / GPTDesync / GPTParallel.
+
+Module tree and public surface follow the reference (gpt_ladder_TP.py:210-288): children
+`tok_embeddings`, `layers`, `norm`, `output`; `setup_caches(max_batch_size, max_seq_length)`;
+`forward(idx [B, S], input_pos [S]) -> logits [B, S, V]`; `from_name`.  forward() is a fixed
+sequence of libladder_hip.so launches over preallocated buffers: no torch kernels, no
+allocation after the first call for a given (B, S), no host synchronisation, positions read from
+the device tensor `input_pos` -- so one decode step can be captured into a hipGraph and replayed
+while `input_pos` and the token buffer are advanced on the device."""
+from typing import Dict, Optional
+
+import torch
+import torch.nn as nn
+from torch import Tensor
+
+from . import _hip
+from .config import ModelArgs, find_multiple
+from .utils import KVCache, RMSNorm, _pos_i32, precompute_freqs_cis
+
+
+class Workspace:
+    """Activation buffers for one (batch, seq) shape, all bf16 [rows, *]."""
+
+    def __init__(self, cfg: ModelArgs, B: int, S: int, fused_width: int, device, dtype, smax: int, all_logits: bool):
+        rows = B * S
+        D, hd = cfg.dim, cfg.head_dim
+        e = lambda *shape: torch.empty(*shape, dtype=dtype, device=device)
+        self.B, self.S, self.rows = B, S, rows
+        self.x = e(rows, D)        # residual stream
+        self.xn = e(rows, D)       # normed input of the current module
+        self.a = e(rows, D)        # attention partial sum (pending in the ladder schedule)
+        self.m = e(rows, D)        # MLP partial sum
+        self.qkv = e(rows, fused_width)
+        self.y = e(rows, cfg.n_head_local * hd)
+        self.h = e(rows, 2 * cfg.ffn_local)
+        self.logits = e(B, S if all_logits else 1, cfg.output_rows)
+        self.next_token = torch.empty(B, 1, dtype=torch.int32, device=device)
+        self.scratch = None
+        if S == 1:
+            n = _hip.attn_decode_scratch_bytes(B, cfg.n_head_local, hd, smax) // 4
+            self.scratch = torch.empty(n, dtype=torch.float32, device=device)
+
+
+class GPTBase(nn.Module):
+    family = "ladder"
+
+    def __init__(self, config: ModelArgs) -> None:
+        super().__init__()
+        self.config = config
+        self.tok_embeddings = nn.Embedding(config.vocab_size, config.dim)
+        self.layers = nn.ModuleList(self._make_block(config, i) for i in range(config.n_layer))
+        self.norm = RMSNorm(config.dim, eps=config.norm_eps)
+        self.output = nn.Linear(config.dim, config.output_rows, bias=False)
+
+        self.freqs_cis: Optional[Tensor] = None
+        self.mask_cache: Optional[Tensor] = None
+        self.causal_mask: Optional[Tensor] = None
+        self.max_batch_size = -1
+        self.max_seq_length = -1
+        # False: logits for every position, as the reference returns; True: only the last position
+        # of each sequence goes through the final norm and lm_head (prefill saves S-1 rows of it)
+        self.last_logits_only = False
+        self._ws: Dict[tuple, Workspace] = {}
+
+    # -- construction ---------------------------------------------------------------------------
+    def _make_block(self, config, layer_idx):
+        raise NotImplementedError
+
+    @classmethod
+    def from_name(cls, name: str):
+        from .config import args_from_name
+
+        return cls(args_from_name(cls.family, name))
+
+    def _fused_width(self) -> int:
+        c = self.config
+        return (c.n_head_local + 2 * c.n_kv_local) * c.head_dim
+
+    # -- caches ---------------------------------------------------------------------------------
+    def setup_caches(self, max_batch_size, max_seq_length):
+        if self.max_seq_length >= max_seq_length and self.max_batch_size >= max_batch_size:
+            return
+        cfg = self.config
+        if cfg.head_dim not in (64, 128):
+            raise NotImplementedError(f"head_dim {cfg.head_dim}: the attention kernels are built for 64 and 128")
+        max_seq_length = find_multiple(max_seq_length, 8)
+        self.max_seq_length = max_seq_length
+        self.max_batch_size = max_batch_size
+        dtype = self.output.weight.dtype
+        device = self.output.weight.device
+        if dtype != torch.bfloat16:
+            raise NotImplementedError(f"the HIP kernels compute in bfloat16 storage; model dtype is {dtype}")
+        for b in self.layers:
+            b.attention.kv_cache = KVCache(max_batch_size, max_seq_length, cfg.n_kv_local, cfg.head_dim, dtype).to(device)
+        self.freqs_cis = precompute_freqs_cis(cfg.block_size, cfg.head_dim, cfg.rope_base, dtype,
+                                              cfg.rope_scaling).to(device)
+        # kept for API compatibility (the kernels derive visibility from input_pos)
+        self.causal_mask = torch.tril(torch.ones(max_seq_length, max_seq_length, dtype=torch.bool, device=device))
+        self._ws.clear()
+
+    def release_workspace(self):
+        self._ws.clear()
+
+    def _workspace(self, B: int, S: int) -> Workspace:
+        key = (B, S, self.last_logits_only)
+        ws = self._ws.get(key)
+        if ws is None:
+            w = self.output.weight
+            ws = Workspace(self.config, B, S, self._fused_width(), w.device, w.dtype, self.max_seq_length,
+                           not self.last_logits_only)
+            if S > 1:  # keep at most one prefill-sized workspace alive
+                for k in [k for k in self._ws if k[1] > 1]:
+                    del self._ws[k]
+            self._ws[key] = ws
+        return ws
+
+    # -- forward --------------------------------------------------------------------------------
+    def forward(self, idx: Tensor, input_pos: Optional[Tensor] = None) -> Tensor:
+        assert self.freqs_cis is not None, "Caches must be initialized first"
+        B, S = idx.shape
+        assert B <= self.max_batch_size and input_pos.shape[-1] == S
+        pos = _pos_i32(input_pos)
+        ws = self._workspace(B, S)
+        _hip.embed(self.tok_embeddings.weight, idx.contiguous(), ws.x)
+        final_d1, final_d2 = self._run_layers(ws, pos)
+        cfg = self.config
+        if self.last_logits_only and S > 1:
+            # only row S-1 of each sequence feeds the head: copy those B rows out, then norm + lm_head
+            last = lambda t: None if t is None else t.view(B, S, -1)[:, S - 1].contiguous()
+            xl = last(ws.x)
+            xn = torch.empty_like(xl)
+            _hip.add_rmsnorm(xl, last(final_d1), last(final_d2), self.norm.weight, None, xn, cfg.norm_eps)
+            _hip.linear(xn, self.output.weight, ws.logits.view(B, -1))
+        else:
+            _hip.add_rmsnorm(ws.x, final_d1, final_d2, self.norm.weight, None, ws.xn, cfg.norm_eps)
+            _hip.linear(ws.xn, self.output.weight, ws.logits.view(B * S, -1))
+        return ws.logits
+
+    def _run_layers(self, ws: Workspace, pos: Tensor):
+        """Runs all blocks on ws.x; returns up to two tensors still to be added to ws.x before the
+        final norm (the ladder's two stragglers), or (None, None)."""
+        raise NotImplementedError
+
+    # -- shared pieces of the block schedules -----------------------------------------------------
+    def _attention(self, ws: Workspace, blk, pos: Tensor, wqkv: Tensor, out: Tensor):
+        """ws.xn -> fused projection -> RoPE + cache write -> attention -> wo -> out (partial sum)."""
+        cfg = self.config
+        B, S = ws.B, ws.S
+        Hq, Hkv, hd = cfg.n_head_local, cfg.n_kv_local, cfg.head_dim
+        kc, vc = blk.attention.kv_cache.k_cache, blk.attention.kv_cache.v_cache
+        _hip.linear(ws.xn, wqkv, ws.qkv)
+        _hip.rope_kv_write(ws.qkv, self.freqs_cis, False, pos, kc, vc, B, S, Hq, Hkv, hd)
+        if S == 1:
+            _hip.attn_decode(ws.qkv, kc, vc, pos, ws.y, ws.scratch, B, Hq, Hkv, hd)
+        else:
+            _hip.attn_prefill(ws.qkv, kc, vc, pos, ws.y, B, S, Hq, Hkv, hd)
+        _hip.linear(ws.y, blk.attention.wo.weight, out)
+
+    def _mlp(self, ws: Workspace, blk, out: Tensor):
+        ff = blk.feed_forward
+        _hip.linear(ws.xn, ff.w1.weight, ws.h)
+        _hip.linear(ws.h, ff.w2.weight, out, act_swiglu=True)
+
+    # -- greedy decoding helper ---------------------------------------------------------------------
+    def greedy_next(self, logits: Tensor) -> Tensor:
+        """argmax of the last position of `logits` [B, S, V] -> int32 [B, 1] (lowest index on ties)."""
+        B = logits.shape[0]
+        ws = self._ws.get((B, 1, self.last_logits_only)) or next(iter(self._ws.values()))
+        out = ws.next_token if ws.next_token.shape[0] == B else torch.empty(B, 1, dtype=torch.int32,
+                                                                            device=logits.device)
+        return _hip.argmax(logits[:, -1], out)

@@ -1,0 +1,295 @@
+"""Per-kernel parity on a real MI355X: every C-ABI entry point of libladder_hip.so against the
+oracle's op (oracle/ladder_oracle.py, eager PyTorch on the same device, same seeded inputs).
+
+Tolerances, all stated in bf16 units-in-the-last-place ("ulp") of the produced tensor:
+  * pure data movement and element-wise work with one rounding (embed, add, RoPE, cache write,
+    argmax, advance): bit-exact;
+  * ops with an fp32 reduction inside (RMSNorm, linear, attention) or a transcendental (SwiGLU):
+    the fp32 value before the final rounding differs from the oracle's by summation order /
+    libm only, so results must agree within 1 ulp and on all but a small fraction of elements."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import ladder_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+BF = torch.bfloat16
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from gpt_fast import _hip
+
+    _hip.load()
+    return _hip
+
+
+def rnd(*shape, seed=0, scale=1.0, dtype=BF):
+    g = torch.Generator(device=DEV)
+    g.manual_seed(seed)
+    return (torch.randn(*shape, generator=g, device=DEV) * scale).to(dtype)
+
+
+def ulp_diff(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """Distance in bf16 steps between two bf16 tensors (monotonic integer mapping of the bits)."""
+    def key(t):
+        i = t.contiguous().view(torch.int16).to(torch.int32)
+        return torch.where(i < 0, -(i & 0x7FFF), i)
+    return (key(a) - key(b)).abs()
+
+
+def assert_close_ulp(got, want, max_ulp=1, max_frac=0.02, what=""):
+    assert got.shape == want.shape and got.dtype == want.dtype == BF
+    assert torch.isfinite(got.float()).all(), what
+    d = ulp_diff(got, want)
+    # values whose magnitude is far below the tensor's scale may differ by many ulps of their own
+    # size while being equal to fp32 accuracy relative to the sum that produced them
+    tiny = want.float().abs() < want.float().abs().max() * 2.0 ** -12
+    bad = (d > max_ulp) & ~tiny
+    frac = (d > 0).float().mean().item()
+    assert not bad.any(), f"{what}: {int(bad.sum())} elements differ by more than {max_ulp} ulp (max {int(d.max())})"
+    assert frac <= max_frac, f"{what}: {frac:.4f} of elements differ (limit {max_frac})"
+
+
+# ------------------------------------------------------------------------------------ embed / add / advance
+
+@pytest.mark.parametrize("idx_dtype", [torch.int64, torch.int32])
+def test_embed_exact(hip, idx_dtype):
+    table = rnd(1000, 512, seed=1)
+    idx = torch.randint(0, 1000, (3, 17), device=DEV, dtype=idx_dtype)
+    out = torch.empty(3 * 17, 512, dtype=BF, device=DEV)
+    hip.embed(table, idx, out)
+    assert torch.equal(out.view(3, 17, 512), F.embedding(idx.long(), table))
+
+
+@pytest.mark.parametrize("n", [8, 2048, 8192 * 5 + 24, 1000003])
+def test_add_exact(hip, n):
+    a, b = rnd(n, seed=2), rnd(n, seed=3)
+    out = torch.empty_like(a)
+    hip.add(a, b, out)
+    assert torch.equal(out, a + b)
+    hip.add(a, b, out, b_div=8.0)
+    assert torch.equal(out, a + b / 8)
+    hip.add(a, b, out, b_div=3.0)
+    assert torch.equal(out, a + b / 3)
+    out2 = b.clone()
+    hip.add(a, out2, out2)  # aliasing the second operand
+    assert torch.equal(out2, a + b)
+
+
+def test_advance_and_history(hip):
+    B = 5
+    cur = torch.zeros(B, 1, dtype=torch.int32, device=DEV)
+    nxt = torch.arange(10, 10 + B, dtype=torch.int32, device=DEV).view(B, 1)
+    pos = torch.tensor([7], dtype=torch.int32, device=DEV)
+    hist = torch.full((B, 4), -1, dtype=torch.int32, device=DEV)
+    hip.advance(cur, nxt, pos, B, hist, pos0=6)
+    assert pos.item() == 8 and torch.equal(cur, nxt) and hist[:, 1].tolist() == list(range(10, 10 + B))
+    assert (hist[:, [0, 2, 3]] == -1).all()
+    hip.advance(None, None, pos, B)
+    assert pos.item() == 9
+
+
+# ------------------------------------------------------------------------------------ RMSNorm
+
+@pytest.mark.parametrize("rows,dim", [(1, 8192), (3, 4096), (64, 8192), (2, 16384), (5, 256), (2048, 2048)])
+def test_add_rmsnorm(hip, rows, dim):
+    r, d1, d2 = rnd(rows, dim, seed=4), rnd(rows, dim, seed=5, scale=0.1), rnd(rows, dim, seed=6, scale=0.1)
+    g = rnd(dim, seed=7, scale=0.02)
+    ro, no = torch.empty_like(r), torch.empty_like(r)
+    # plain norm
+    hip.add_rmsnorm(r, None, None, g, None, no, 1e-5)
+    # two roundings in a row (normalised value, then gain product): a 1-ulp flip of the first can
+    # show as 2 ulp after the second, hence max_ulp=2 for this op only
+    assert_close_ulp(no, O.rms_norm(r, g, 1e-5), max_ulp=2, max_frac=0.01, what="norm")
+    # one pending partial (ladder add), residual written back
+    hip.add_rmsnorm(r, d1, None, g, ro, no, 1e-5)
+    assert torch.equal(ro, r + d1)
+    assert_close_ulp(no, O.rms_norm(r + d1, g, 1e-5), max_ulp=2, max_frac=0.01, what="add+norm")
+    # two pending partials (closing add of the ladder), in place
+    r2 = r.clone()
+    hip.add_rmsnorm(r2, d1, d2, g, r2, no, 1e-5)
+    assert torch.equal(r2, r + d1 + d2)
+    assert_close_ulp(no, O.rms_norm(r + d1 + d2, g, 1e-5), max_ulp=2, max_frac=0.01, what="add+add+norm")
+
+
+# ------------------------------------------------------------------------------------ linear
+
+def linear_ref(x, w):
+    """fp64 product rounded once: what any fp32-accumulating bf16 linear must match within 1 ulp."""
+    return (x.double() @ w.double().T).to(BF)
+
+
+GEMV_SHAPES = [  # (N, K): the 70B rank shard, the 8B model, the 1B model, and ragged sizes
+    (1280, 8192), (8192, 1024), (7168, 8192), (8192, 3584), (16032, 8192),
+    (6144, 4096), (4096, 4096), (3072, 2048), (2048, 8192), (24, 64), (1001, 520),
+]
+
+
+@pytest.mark.parametrize("N,K", GEMV_SHAPES)
+@pytest.mark.parametrize("M", [1, 2, 3, 5, 8])
+def test_linear_gemv(hip, M, N, K):
+    if M in (2, 3, 5) and N * K > 20e6:
+        pytest.skip("odd batch sizes are covered on the smaller shapes")
+    x = rnd(M, K, seed=8)
+    w = rnd(N, K, seed=9, scale=0.02)
+    y = torch.empty(M, N, dtype=BF, device=DEV)
+    hip.linear(x, w, y)
+    assert_close_ulp(y, linear_ref(x, w), what=f"gemv M={M} N={N} K={K}")
+    # and against the library routine the reference uses
+    assert_close_ulp(y, F.linear(x, w), max_frac=0.05, what="gemv vs F.linear")
+
+
+@pytest.mark.parametrize("cfg", [144, 212, 222, 242, 244, 412, 422, 442])
+def test_linear_gemv_every_launch_configuration(hip, cfg):
+    x = rnd(4, 3584, seed=10)
+    w = rnd(1030, 3584, seed=11, scale=0.02)
+    y = torch.empty(4, 1030, dtype=BF, device=DEV)
+    lib = hip.load()
+    try:
+        lib.lr_gemv_set_cfg(cfg)
+        hip.linear(x, w, y)
+    finally:
+        lib.lr_gemv_set_cfg(0)
+    assert_close_ulp(y, linear_ref(x, w), what=f"gemv cfg {cfg}")
+
+
+def test_linear_gemv_is_deterministic(hip):
+    x = rnd(1, 8192, seed=12)
+    w = rnd(1280, 8192, seed=13, scale=0.02)
+    ys = []
+    for _ in range(5):
+        y = torch.empty(1, 1280, dtype=BF, device=DEV)
+        hip.linear(x, w, y)
+        ys.append(y)
+    assert all(torch.equal(ys[0], t) for t in ys[1:])
+
+
+@pytest.mark.parametrize("M,N,K", [(9, 256, 64), (128, 128, 64), (130, 1280, 8192), (2048, 1280, 1024),
+                                   (333, 1001, 520), (64, 16032, 2048), (16, 8192, 3584), (257, 384, 8)])
+def test_linear_gemm(hip, M, N, K):
+    x = rnd(M, K, seed=14)
+    w = rnd(N, K, seed=15, scale=0.02)
+    y = torch.empty(M, N, dtype=BF, device=DEV)
+    hip.linear(x, w, y)
+    assert_close_ulp(y, linear_ref(x, w), what=f"gemm M={M} N={N} K={K}")
+
+
+def test_linear_strided_rows(hip):
+    big = rnd(6, 3 * 512, seed=16)
+    x = big[:, 512:1024]                      # row stride 1536
+    w = rnd(200, 512, seed=17, scale=0.05)
+    out = torch.zeros(6, 2 * 200, dtype=BF, device=DEV)
+    y = out[:, 200:]                          # row stride 400
+    hip.linear(x, w, y)
+    assert_close_ulp(y.contiguous(), linear_ref(x, w), what="strided")
+    assert (out[:, :200] == 0).all()
+
+
+@pytest.mark.parametrize("rows", [1, 4, 8, 40])
+def test_swiglu_and_fused_w2(hip, rows):
+    I, D = 3584, 1024
+    h = rnd(rows, 2 * I, seed=18)
+    w2 = rnd(D, I, seed=19, scale=0.02)
+    u, g = h.chunk(2, dim=-1)
+    act = F.silu(g) * u
+    out = torch.empty(rows, I, dtype=BF, device=DEV)
+    hip.swiglu(h, out)
+    assert_close_ulp(out, act, max_frac=0.002, what="swiglu")
+    y = torch.empty(rows, D, dtype=BF, device=DEV)
+    hip.linear(h, w2, y, act_swiglu=True)
+    assert_close_ulp(y, linear_ref(act, w2), max_frac=0.05, what="w2(silu(g)*u)")
+
+
+# ------------------------------------------------------------------------------------ RoPE + cache
+
+@pytest.mark.parametrize("hd,Hq,Hkv", [(128, 8, 1), (64, 32, 8), (128, 32, 8)])
+@pytest.mark.parametrize("gathered", [False, True])
+def test_rope_kv_write_exact(hip, hd, Hq, Hkv, gathered):
+    B, S, Smax, block = 2, 9, 32, 64
+    width = (Hq + 2 * Hkv) * hd
+    qkv = rnd(B, S, width + 16, seed=20)[..., :width]          # padded rows: row stride != width
+    pos = torch.tensor([3, 4, 5, 6, 7, 8, 9, 20, 31], dtype=torch.int32, device=DEV)
+    table = O.rope_table(block, hd, 500000, BF).to(DEV)
+    kc = torch.zeros(B + 1, Hkv, Smax, hd, dtype=BF, device=DEV)
+    vc = torch.zeros_like(kc)
+    q, k, v = qkv.clone().split([Hq * hd, Hkv * hd, Hkv * hd], dim=-1)
+    fc = table[pos.long()]
+    q_ref = O.apply_rope(q.reshape(B, S, Hq, hd), fc)
+    k_ref = O.apply_rope(k.reshape(B, S, Hkv, hd), fc).transpose(1, 2)
+    kc_ref, vc_ref = kc.clone(), vc.clone()
+    O.kv_update(kc_ref, vc_ref, pos.long(), k_ref, v.reshape(B, S, Hkv, hd).transpose(1, 2))
+
+    work = qkv  # rotated in place on the strided view
+    hip.rope_kv_write(work, fc.contiguous() if gathered else table, gathered, pos, kc, vc, B, S, Hq, Hkv, hd)
+    assert torch.equal(work[..., : Hq * hd].reshape(B, S, Hq, hd), q_ref)
+    assert torch.equal(kc, kc_ref) and torch.equal(vc, vc_ref)
+    assert torch.equal(work[..., Hq * hd:], torch.cat([k, v], -1))   # k and v columns are left as they were
+
+
+# ------------------------------------------------------------------------------------ attention
+
+@pytest.mark.parametrize("B,Hq,Hkv,hd,Smax,pos", [
+    (1, 8, 1, 128, 2176, 2048), (1, 8, 1, 128, 2176, 0), (1, 8, 1, 128, 2176, 2175), (8, 8, 1, 128, 2176, 2100),
+    (64, 8, 1, 128, 2176, 2111), (2, 32, 8, 128, 1280, 1033), (1, 32, 8, 64, 160, 131), (16, 16, 1, 128, 4160, 4100),
+    (3, 4, 4, 64, 40, 17), (2, 8, 4, 128, 264, 200), (1, 16, 1, 128, 520, 519),
+])
+def test_attn_decode(hip, B, Hq, Hkv, hd, Smax, pos):
+    q = rnd(B, Hq * hd, seed=21)
+    kc = rnd(B, Hkv, Smax, hd, seed=22)
+    vc = rnd(B, Hkv, Smax, hd, seed=23)
+    kc[:, :, pos + 1:] = 7.0   # garbage beyond pos must not be read
+    vc[:, :, pos + 1:] = -9.0
+    p = torch.tensor([pos], dtype=torch.int32, device=DEV)
+    y = torch.empty(B, Hq * hd, dtype=BF, device=DEV)
+    scratch = torch.empty(hip.attn_decode_scratch_bytes(B, Hq, hd, Smax) // 4, dtype=torch.float32, device=DEV)
+    hip.attn_decode(q, kc, vc, p, y, scratch, B, Hq, Hkv, hd)
+    mask = (torch.arange(Smax, device=DEV) <= pos).view(1, Smax)
+    want = O.sdpa_math(q.view(B, 1, Hq, hd).transpose(1, 2), kc, vc, mask).transpose(1, 2).reshape(B, Hq * hd)
+    assert_close_ulp(y, want, max_frac=0.03, what="attn_decode")
+
+
+@pytest.mark.parametrize("B,S,Hq,Hkv,hd,Smax,start", [
+    (1, 128, 8, 1, 128, 136, 0), (2, 100, 4, 2, 64, 160, 0), (1, 300, 8, 1, 128, 512, 100), (1, 2048, 8, 1, 128, 2176, 0),
+    (3, 65, 32, 8, 64, 72, 0),
+])
+def test_attn_prefill(hip, B, S, Hq, Hkv, hd, Smax, start):
+    q = rnd(B, S, Hq * hd, seed=24)
+    kc = rnd(B, Hkv, Smax, hd, seed=25)
+    vc = rnd(B, Hkv, Smax, hd, seed=26)
+    pos = torch.arange(start, start + S, dtype=torch.int32, device=DEV)
+    y = torch.empty(B, S, Hq * hd, dtype=BF, device=DEV)
+    hip.attn_prefill(q, kc, vc, pos, y, B, S, Hq, Hkv, hd)
+    mask = torch.arange(Smax, device=DEV).view(1, Smax) <= pos.view(S, 1)
+    want = O.sdpa_math(q.view(B, S, Hq, hd).transpose(1, 2), kc, vc, mask).transpose(1, 2).reshape(B, S, Hq * hd)
+    assert_close_ulp(y, want, max_frac=0.03, what="attn_prefill")
+
+
+# ------------------------------------------------------------------------------------ argmax
+
+def test_argmax_lowest_index_on_ties(hip):
+    B, V = 4, 128256
+    lg = rnd(B, V, seed=27, scale=0.04)
+    lg[0, [77, 100000]] = 5.0
+    lg[1, [128255, 5]] = 5.0
+    lg[2, 128255] = 9.0
+    out = torch.empty(B, 1, dtype=torch.int32, device=DEV)
+    hip.argmax(lg, out)
+    want = torch.argmax(lg, dim=-1, keepdim=True).to(torch.int32)
+    assert torch.equal(out, want) and out.flatten().tolist()[:3] == [77, 5, 128255]
+    # last position of [B, S, V] logits: a strided [B, V] view; and a vocab that is not a multiple of 8
+    lg3 = rnd(2, 3, 1008, seed=28)
+    hip.argmax(lg3[:, -1, :1003], out[:2])
+    assert torch.equal(out[:2], lg3[:, -1, :1003].argmax(-1, keepdim=True).to(torch.int32))
+
+
+def test_torch_argmax_itself_returns_first_maximum_on_this_device():
+    """The oracle's greedy() relies on it."""
+    lg = torch.zeros(1, 16032, dtype=BF, device=DEV)
+    lg[0, [15000, 40, 9000]] = 1.0
+    assert torch.argmax(lg, -1).item() == 40
