@@ -1,0 +1,171 @@
+"""Headline benchmark: batch-1 greedy decode of one TP=8 rank shard of Ladder-70B on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--no-cpu-baseline]
+
+A "step" is one decode step (one new token per sequence) of the whole per-rank forward pass,
+replayed as a captured hipGraph: embedding -> 80 ladder blocks -> final add/norm -> vocab-shard
+lm_head -> argmax -> device-side token/position hand-over.  Weights are random N(0, 0.02) bf16
+(seed 0), the prompt is 2048 uniform-random ids; the prompt is prefilled before the timed region
+so the KV cache has its real length, and the timed steps start at position 2048.  Everything the
+steps read is resident in HBM when the clock starts.
+
+Prints ONE JSON line.  `value` = decoded tokens per second (whole job = the one GPU).
+`roofline`   : the dominant kernel, the weight-streaming GEMV on the w1 (up+gate) projection
+               [7168 x 8192] -- 47 % of a step's bytes.  `achieved` = its algorithmic bytes per launch
+               (weight matrix + input row(s) + output row(s)) / its mean launch duration, measured
+               here with HIP events around 80 back-to-back launches over the 80 layers' distinct
+               matrices (so nothing is served from cache) on the launch stream.
+`step_roofline`: the same ratio for the whole decode step: algorithmic bytes per step (all weights
+               and gains once + valid KV + KV write + embedding rows) / measured step time.
+`cpu_baseline`: the oracle (a PyTorch-CPU restatement of the reference; the reference itself cannot
+               run without CUDA + NCCL) timed on this machine's host cores on the reference's
+               CPU-sized case: Ladder-1B fp32, batch 1, 128-token prompt, greedy decode."""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "ladder-residual-inference_amd"))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def cpu_baseline(new_tokens=32, repeats=2):
+    """Oracle on the host cores, config 1 of the benchmark set.  Returns the cpu_baseline object."""
+    import torch
+
+    from oracle import ladder_oracle as O
+
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    torch.set_num_threads(cores)
+    cfg = O.OracleConfig(block_size=2048, vocab_size=128256, n_layer=16, n_head=32, n_local_heads=8, dim=2048,
+                         intermediate_size=8192, rope_base=500000)
+    dev = "cuda" if torch.cuda.is_available() else "cpu"   # generate the random weights fast, compute on the CPU
+    P = {k: v.float().cpu() for k, v in O.init_params(cfg, seed=0, dtype=torch.float32, device=dev).items()}
+    g = torch.Generator()
+    g.manual_seed(1)
+    prompt = torch.randint(0, cfg.vocab_size, (128,), generator=g)
+    O.generate(cfg, P, prompt, 2, 1)  # warm the allocator and thread pool
+    dec, pre = [], []
+    for _ in range(repeats):
+        tm = {}
+        O.generate(cfg, P, prompt, new_tokens, 1, timers=tm)
+        dec.append(tm["decode_latency"] / (new_tokens - 1))
+        pre.append(tm["prefill_latency"])
+    ms = 1e3 * sum(dec) / len(dec)
+    return {"value": round(1e3 / ms, 3), "unit": "tok/s", "cores": cores, "kind": "port",
+            "ms_per_token": round(ms, 3), "prefill_s": round(sum(pre) / len(pre), 3),
+            "sample": f"oracle (PyTorch CPU fp32) on Ladder-1B (dim 2048, 16 layers, 32q/8kv, FFN 8192, vocab 128256), "
+                      f"B=1, prompt 128, greedy decode of {new_tokens} tokens, {repeats} runs"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=127)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--prompt", type=int, default=2048)
+    ap.add_argument("--model", type=str, default="gpt_ladder:ladder-70b-tp8")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures ONE tensor-parallel rank's shard on ONE GPU (partial sums stay local, no "
+              "collectives); --gpus must be 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import benchmark as bm
+    from gpt_fast import _hip
+
+    assert torch.cuda.is_available(), "bench.py needs the MI355X"
+    _hip.load()
+    dev = "cuda"
+    B, T, K, W = args.batch, args.prompt, args.steps, args.warmup
+    model = bm._load_model(args.model, dev, torch.bfloat16, seed=0, verbose=False)
+    model.last_logits_only = True          # prefill is set-up here, not the timed region
+    cfg = model.config
+    new = max(K, W, 127) + 1
+    g = torch.Generator(device=dev)
+    g.manual_seed(1)
+    prompt = torch.randint(0, cfg.vocab_size, (T,), device=dev, generator=g)
+    model.setup_caches(B, T + new)
+
+    # ---- set-up: prefill the prompt (eager), capture the decode step
+    rows = prompt.view(1, -1).repeat(B, 1)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    first = bm.prefill(model, rows, torch.arange(T, device=dev, dtype=torch.int32), greedy=True).clone()
+    torch.cuda.synchronize()
+    prefill_s = time.perf_counter() - t0
+    dg = bm.get_cuda_graphs_for_decode(model, prompt, B, new, first, greedy=True)
+
+    # ---- W untimed steps, then exactly K timed steps from position T
+    dg.reset(first)
+    for _ in range(W):
+        dg.replay()
+    dg.reset(first)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(K):
+        dg.replay()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = 1e3 * elapsed / K
+    tokens = dg.history[0, : min(K, 16)].tolist()
+
+    step_bytes = sum(bm.decode_bytes_per_step(cfg, B, T + i) for i in range(K)) / K
+    step_gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # ---- dominant kernel: w1 GEMV, HIP events on the launch stream, distinct matrix per launch
+    w1s = [blk.feed_forward.w1.weight for blk in model.layers] if hasattr(model.layers[0], "feed_forward") else \
+        [blk.attention.wqkv1.weight for blk in model.layers]
+    N, Kdim = w1s[0].shape
+    x = torch.randn(B, Kdim, device=dev).to(torch.bfloat16)
+    y = torch.empty(B, N, device=dev, dtype=torch.bfloat16)
+    for w in w1s[:8]:
+        _hip.linear(x, w, y)
+    reps = 3
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    ev0.record()
+    for _ in range(reps):
+        for w in w1s:
+            _hip.linear(x, w, y)
+    ev1.record()
+    torch.cuda.synchronize()
+    gemv_us = 1e3 * ev0.elapsed_time(ev1) / (reps * len(w1s))
+    gemv_bytes = 2 * (N * Kdim + B * Kdim + B * N)
+    gemv_gbps = gemv_bytes / (gemv_us * 1e-6) / 1e9
+
+    out = {
+        "metric": "decode_tokens_per_sec", "value": round(B * 1e3 / ms_per_step, 2), "unit": "tok/s",
+        "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{args.model} rank shard (dim {cfg.dim}, {cfg.n_layer} layers, {cfg.n_head_local} q / "
+                               f"{cfg.n_kv_local} kv heads, FFN {cfg.ffn_local}, lm_head rows {cfg.output_rows}), "
+                               f"batch {B}, prompt {T}, greedy decode, hipGraph replay per step",
+                   "batch": B, "prompt_len": T, "virtual_tp": cfg.tp_world_size},
+        "ms_per_token": round(ms_per_step, 4),
+        "prefill_s": round(prefill_s, 4),
+        "roofline": {"bound": "hbm", "kernel": f"k_gemv (w1 up+gate projection, [{N} x {Kdim}] bf16, M={B})",
+                     "achieved": round(gemv_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gemv_gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "bytes_per_launch": gemv_bytes, "avg_launch_us": round(gemv_us, 3)},
+        "step_roofline": {"bound": "hbm", "achieved": round(step_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                          "frac": round(step_gbps / HBM_PEAK_GBPS, 4), "bytes_per_step": int(step_bytes)},
+        "first_tokens": tokens,
+    }
+    if not args.no_cpu_baseline:
+        del dg, model
+        torch.cuda.empty_cache()
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()
