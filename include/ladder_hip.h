@@ -127,6 +127,50 @@ int lr_argmax(const void* logits, int64_t ldl, int32_t* out, int B, int V, lr_st
 int lr_advance(int32_t* cur_token, const int32_t* next_token, int32_t* pos, int B, int32_t* history, int64_t ld_hist,
                int hist_len, int pos0, lr_stream_t stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * One whole decode step of the Ladder model as a single persistent kernel (batch 1 or 2).
+ * Replaces, for S == 1, the body of GPTLadder.forward (gpt_ladder_TP.py:252-284: embedding, the
+ * n_layer LadderTransformerBlock.forward calls :312-358 with every op inside them, the closing
+ * x + prev_attn + prev_mlp, final norm, lm_head) plus the greedy token choice and the
+ * between-steps bookkeeping of generate_using_cuda_graphs (benchmark.py:208-217).
+ * All sizes in lr_ladder_model_t are THIS RANK's (already divided by the tensor-parallel size). */
+typedef struct {
+  const void *wqkv, *wo, *w1, *w2, *attention_norm, *ffn_norm; /* bf16 weights of one layer        */
+  void *k_cache, *v_cache;                                     /* [Bmax, n_kv_head, smax, head_dim] */
+} lr_layer_t;
+
+typedef struct {
+  int32_t dim, n_layer, n_head, n_kv_head, head_dim, ffn, out_rows, vocab, smax, block_size;
+  float eps;
+  const void *tok_embeddings, *norm, *output, *freqs_cis; /* [vocab, dim], [dim], [out_rows, dim], table */
+  const lr_layer_t* layers_dev;                           /* DEVICE array of n_layer entries            */
+} lr_ladder_model_t;
+
+/* Bytes of device workspace the step needs (0: shape not supported by the fused step; callers
+ * then use the per-op entry points).  The workspace must be 256-byte aligned, must be
+ * initialised once with lr_ladder_step_init before the first step and belongs to one model. */
+size_t lr_ladder_step_workspace_bytes(const lr_ladder_model_t* model, int batch);
+int lr_ladder_step_init(const lr_ladder_model_t* model, int batch, void* workspace, size_t bytes, lr_stream_t stream);
+
+/* logits[b, :] (bf16, row stride ldl) = model(tokens[b], position pos[0]) and
+ * next_token[b] = argmax (lowest index on ties; may be NULL).  K/V of the new position are written
+ * to the caches.  If advance != 0 the step also performs, on the device,
+ *     history[b, pos[0] - pos0] = next_token[b] (if history),  cur_token[b] = next_token[b] (if
+ *     cur_token),  pos[0] += 1,
+ * so that replaying the captured step is a complete decode loop.  tokens and cur_token may alias.
+ * The kernel occupies every CU and synchronises them with device-wide barriers: nothing else may
+ * run on the device concurrently, and two steps must not overlap.  Barrier waits are bounded; if
+ * one ever expires the workspace word at lr_ladder_step_fail_offset() becomes non-zero, the
+ * outputs of that step are undefined and the workspace must be initialised again. */
+int lr_ladder_decode_step(const lr_ladder_model_t* model, int batch, const int32_t* tokens, int32_t* pos, void* logits,
+                          int64_t ldl, int32_t* next_token, int advance, int32_t* cur_token, int32_t* history,
+                          int64_t ld_hist, int hist_len, int pos0, void* workspace, size_t bytes, lr_stream_t stream);
+size_t lr_ladder_step_fail_offset(void);
+
+/* Tuning hook, no counterpart in the reference: w1 row pairs per workgroup handled in the first
+ * phase of a slot (the rest run beside attention); negative restores the built-in balance. */
+void lr_ladder_step_tune(int p1_pairs_per_wg);
+
 /* Tuning hook, no counterpart in the reference: force the GEMV launch configuration
  * (rows-per-wave * 100 + K-split * 10 + unroll; 0 restores the built-in shape heuristic).
  * Results do not depend on it beyond fp32 summation order. */

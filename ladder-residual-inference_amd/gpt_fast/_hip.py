@@ -32,7 +32,20 @@ _PROTOS = {
     "lr_argmax": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_int, c_void_p]),
     "lr_advance": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "lr_gemv_set_cfg": (None, [c_int]),
+    "lr_ladder_step_workspace_bytes": (c_size_t, [c_void_p, c_int]),
+    "lr_ladder_step_init": (c_int, [c_void_p, c_int, c_void_p, c_size_t, c_void_p]),
+    "lr_ladder_decode_step": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_void_p,
+                                      c_void_p, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "lr_ladder_step_fail_offset": (c_size_t, []),
+    "lr_ladder_step_tune": (None, [c_int]),
 }
+
+
+class LadderModelDesc(ctypes.Structure):
+    """lr_ladder_model_t of include/ladder_hip.h (per-rank sizes)."""
+    _fields_ = [(n, c_int32) for n in ("dim", "n_layer", "n_head", "n_kv_head", "head_dim", "ffn", "out_rows", "vocab",
+                                       "smax", "block_size")] + [("eps", c_float)] + \
+               [(n, c_void_p) for n in ("tok_embeddings", "norm", "output", "freqs_cis", "layers_dev")]
 
 
 class LadderHipError(RuntimeError):
@@ -193,3 +206,64 @@ def advance(cur_token, next_token, pos, B, history=None, pos0=0):
     ld, n = (history.stride(0), history.shape[1]) if history is not None else (0, 0)
     _check(load().lr_advance(p(cur_token), p(next_token), p(pos), B, p(history), ld, n, int(pos0), _stream()),
            "lr_advance")
+
+
+class FusedLadderStep:
+    """Device-side state of lr_ladder_decode_step for one model and batch size: the layer pointer
+    table, the model descriptor and the (initialised) workspace.  Keeps references to every tensor
+    whose address it handed to the library."""
+
+    def __init__(self, model, batch: int):
+        cfg = model.config
+        dev = model.output.weight.device
+        rows = []
+        self._keep = []
+        for blk in model.layers:
+            ts = [blk.attention.wqkv.weight, blk.attention.wo.weight, blk.feed_forward.w1.weight,
+                  blk.feed_forward.w2.weight, blk.attention_norm.weight, blk.ffn_norm.weight,
+                  blk.attention.kv_cache.k_cache, blk.attention.kv_cache.v_cache]
+            for t in ts:
+                assert t.is_contiguous() and t.dtype == torch.bfloat16 and t.device == dev
+            self._keep.append(ts)
+            rows.append([t.data_ptr() for t in ts])
+        self.layer_table = torch.tensor(rows, dtype=torch.int64).to(dev)
+        self._keep += [model.tok_embeddings.weight, model.norm.weight, model.output.weight, model.freqs_cis]
+        self.desc = LadderModelDesc(
+            dim=cfg.dim, n_layer=cfg.n_layer, n_head=cfg.n_head_local, n_kv_head=cfg.n_kv_local, head_dim=cfg.head_dim,
+            ffn=cfg.ffn_local, out_rows=cfg.output_rows, vocab=cfg.vocab_size, smax=model.max_seq_length,
+            block_size=cfg.block_size, eps=cfg.norm_eps, tok_embeddings=model.tok_embeddings.weight.data_ptr(),
+            norm=model.norm.weight.data_ptr(), output=model.output.weight.data_ptr(),
+            freqs_cis=model.freqs_cis.data_ptr(), layers_dev=self.layer_table.data_ptr())
+        self.batch = batch
+        lib = load()
+        self.bytes = int(lib.lr_ladder_step_workspace_bytes(ctypes.byref(self.desc), batch))
+        self.supported = self.bytes > 0
+        self.workspace = None
+        if self.supported:
+            self.workspace = torch.empty(self.bytes + 256, dtype=torch.uint8, device=dev)
+            off = (-self.workspace.data_ptr()) % 256
+            self.workspace = self.workspace[off:off + self.bytes]
+            self.reset()
+
+    def reset(self):
+        _check(load().lr_ladder_step_init(ctypes.byref(self.desc), self.batch, self.workspace.data_ptr(), self.bytes,
+                                          _stream()), "lr_ladder_step_init")
+
+    def failed(self) -> bool:
+        """Synchronises.  True if a barrier wait of an earlier step expired."""
+        off = int(load().lr_ladder_step_fail_offset())
+        return bool(self.workspace[off:off + 4].view(torch.int32).item())
+
+    def step(self, tokens, pos, logits, next_token=None, advance=False, cur_token=None, history=None, pos0=0):
+        B = self.batch
+        for t in (tokens, pos, next_token, cur_token, history):
+            assert t is None or (t.dtype == torch.int32 and t.is_cuda)
+        assert tokens.numel() == B and pos.numel() == 1 and logits.dtype == torch.bfloat16
+        lrows, lcols, ldl = _rows_ld(logits)
+        assert lrows == B and lcols == self.desc.out_rows
+        p = lambda t: None if t is None else t.data_ptr()
+        ld, n = (history.stride(0), history.shape[1]) if history is not None else (0, 0)
+        _check(load().lr_ladder_decode_step(ctypes.byref(self.desc), B, tokens.data_ptr(), pos.data_ptr(),
+                                            logits.data_ptr(), ldl, p(next_token), int(bool(advance)), p(cur_token),
+                                            p(history), ld, n, int(pos0), self.workspace.data_ptr(), self.bytes,
+                                            _stream()), "lr_ladder_decode_step")

@@ -35,6 +35,7 @@ class Workspace:
         self.h = e(rows, 2 * cfg.ffn_local)
         self.logits = e(B, S if all_logits else 1, cfg.output_rows)
         self.next_token = torch.empty(B, 1, dtype=torch.int32, device=device)
+        self.next_token_valid_for = None   # set by a fused decode step that already chose the token
         self.scratch = None
         if S == 1:
             n = _hip.attn_decode_scratch_bytes(B, cfg.n_head_local, hd, smax) // 4
@@ -121,6 +122,7 @@ class GPTBase(nn.Module):
         assert B <= self.max_batch_size and input_pos.shape[-1] == S
         pos = _pos_i32(input_pos)
         ws = self._workspace(B, S)
+        ws.next_token_valid_for = None
         _hip.embed(self.tok_embeddings.weight, idx.contiguous(), ws.x)
         final_d1, final_d2 = self._run_layers(ws, pos)
         cfg = self.config

@@ -58,9 +58,58 @@ class LadderTransformerBlock(nn.Module):
 
 class GPTLadder(GPTBase):
     family = "ladder"
+    # decode steps of batch <= 2 run as ONE persistent kernel (lr_ladder_decode_step) when the shape
+    # is supported; set to False to force the per-op kernels
+    use_fused_step = True
 
     def _make_block(self, config, layer_idx):
         return LadderTransformerBlock(config)
+
+    def setup_caches(self, max_batch_size, max_seq_length):
+        before = self.max_seq_length, self.max_batch_size
+        super().setup_caches(max_batch_size, max_seq_length)
+        if (self.max_seq_length, self.max_batch_size) != before:
+            self._fused = {}
+
+    def _fused_step(self, B: int):
+        st = getattr(self, "_fused", None)
+        if st is None:
+            st = self._fused = {}
+        if B not in st:
+            st[B] = _hip.FusedLadderStep(self, B) if B <= 2 else None
+            if st[B] is not None and not st[B].supported:
+                st[B] = None
+        return st[B]
+
+    def forward(self, idx: Tensor, input_pos=None) -> Tensor:
+        B, S = idx.shape
+        if S == 1 and self.use_fused_step and B <= 2 and self.freqs_cis is not None:
+            fused = self._fused_step(B)
+            if fused is not None:
+                return self.decode_step_fused(idx, input_pos)
+        return super().forward(idx, input_pos)
+
+    def decode_step_fused(self, idx: Tensor, input_pos: Tensor, advance: bool = False, history=None, pos0: int = 0):
+        """One decode step through lr_ladder_decode_step.  Returns logits [B, 1, V]; the greedy token
+        is left in the workspace's next_token buffer (see greedy_next).  With advance=True the step
+        also writes the token into `idx` (must be int32), `history[:, pos - pos0]`, and bumps
+        `input_pos` (must be int32) on the device."""
+        B = idx.shape[0]
+        fused = self._fused_step(B)
+        ws = self._workspace(B, 1)
+        tokens = idx if idx.dtype == torch.int32 else idx.to(torch.int32)
+        pos = input_pos if input_pos.dtype == torch.int32 else input_pos.to(torch.int32)
+        assert not advance or (tokens is idx and pos is input_pos), "advance needs int32 token and position buffers"
+        fused.step(tokens.contiguous(), pos, ws.logits.view(B, -1), ws.next_token, advance,
+                   tokens if advance else None, history, pos0)
+        ws.next_token_valid_for = ws.logits
+        return ws.logits
+
+    def greedy_next(self, logits: Tensor) -> Tensor:
+        ws = self._ws.get((logits.shape[0], 1, self.last_logits_only))
+        if ws is not None and getattr(ws, "next_token_valid_for", None) is logits:
+            return ws.next_token  # already chosen inside the fused step
+        return super().greedy_next(logits)
 
     def _run_layers(self, ws: Workspace, pos: Tensor):
         eps = self.config.norm_eps

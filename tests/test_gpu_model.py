@@ -58,10 +58,14 @@ def near_tie_ok(ref_logits, tok, ulps=2):
 
 
 @torch.no_grad()
-def run_parity(model, family, B, T, new, seed=1, check_graph=True):
-    """Prefill + (new - 1) decode steps, HIP vs oracle.  Returns a dict of statistics."""
+def run_parity(model, family, B, T, new, seed=1, check_graph=True, fused=None):
+    """Prefill + (new - 1) decode steps, HIP vs oracle.  Returns a dict of statistics.
+    fused: True / False selects the persistent one-kernel decode step or the per-op kernels for the
+    ladder family at batch <= 2 (None: the model's default)."""
     import benchmark as bm
 
+    if fused is not None:
+        model.use_fused_step = fused
     cfg = model.config
     ocfg = oracle_cfg(cfg)
     P = dict(model.state_dict())          # the very same device tensors
@@ -110,6 +114,10 @@ def run_parity(model, family, B, T, new, seed=1, check_graph=True):
             dg.replay()
         torch.cuda.synchronize()
         stats["graph_equals_eager"] = bool(torch.equal(dg.history[:, : new - 1], free[:, 1:]))
+    fs = getattr(model, "_fused", {}).get(B) if getattr(model, "use_fused_step", False) else None
+    stats["fused_step_used"] = fs is not None
+    if fs is not None:
+        assert not fs.failed(), "a device-wide barrier of the fused decode step timed out"
     return stats
 
 
@@ -123,6 +131,24 @@ def check(stats, min_exact=0.7):
 
 TINY = dict(block_size=64, vocab_size=512, n_layer=3, n_head=4, n_local_heads=2, dim=256, intermediate_size=512,
             rope_base=10000)
+
+
+@pytest.mark.parametrize("B", [1, 2])
+@pytest.mark.parametrize("fused", [True, False])
+def test_tiny_ladder_fused_and_per_op_decode(B, fused):
+    stats = run_parity(build("ladder", **TINY), "ladder", B=B, T=20, new=12, fused=fused)
+    print(B, fused, stats)
+    check(stats)
+    assert stats["fused_step_used"] == fused
+
+
+def test_tiny_ladder_fused_head_dim_128_many_kv_heads():
+    kw = dict(TINY, block_size=128, n_head=8, n_local_heads=2, dim=1024, intermediate_size=768, n_layer=2,
+              vocab_size=1000)
+    stats = run_parity(build("ladder", **kw), "ladder", B=2, T=70, new=10, fused=True)
+    print(stats)
+    check(stats)
+    assert stats["fused_step_used"]
 
 
 @pytest.mark.parametrize("family", ["ladder", "dense", "desync", "parallel"])
@@ -219,7 +245,14 @@ def test_ladder_1b_config1_full():
     check(stats)
 
 
-@pytest.mark.parametrize("B,layers,T,new", [(1, 80, 2048, 128), (8, 16, 2048, 24), (64, 4, 512, 6)])
+def test_ladder_70b_tp8_shard_per_op_kernels_b1():
+    stats = run_parity(build("ladder", **shape_kw("ladder-70b-tp8", 12)), "ladder", B=1, T=2048, new=24, fused=False)
+    print(stats)
+    check(stats)
+    assert not stats["fused_step_used"]
+
+
+@pytest.mark.parametrize("B,layers,T,new", [(1, 80, 2048, 128), (2, 10, 2048, 16), (8, 16, 2048, 24), (64, 4, 512, 6)])
 def test_ladder_70b_tp8_shard(B, layers, T, new):
     """Config 3: one TP=8 rank shard of Ladder-70B (dim 8192, 8 q / 1 kv heads, FFN 3584, vocab shard
     16032).  B=1 runs the full 80 layers at the full prompt and decode length; the larger batches
