@@ -167,9 +167,15 @@ int lr_ladder_decode_step(const lr_ladder_model_t* model, int batch, const int32
                           int64_t ld_hist, int hist_len, int pos0, void* workspace, size_t bytes, lr_stream_t stream);
 size_t lr_ladder_step_fail_offset(void);
 
-/* Tuning hook, no counterpart in the reference: w1 row pairs per workgroup handled in the first
- * phase of a slot (the rest run beside attention); negative restores the built-in balance. */
-void lr_ladder_step_tune(int p1_pairs_per_wg);
+/* Tuning hook, no counterpart in the reference: use at least this many attention workgroups in
+ * the step kernel (more workgroups, fewer keys each; <= 0 restores the default).  Set it before the
+ * workspace is sized and initialised. */
+void lr_ladder_step_tune(int attention_workgroups);
+
+/* Debug hook, no counterpart in the reference: following steps record, per workgroup, up to 12 wall-clock
+ * stamps (100 MHz) for 4 consecutive slots starting at `first_slot` into `device_buffer` (NULL
+ * switches it off).  Returns the bytes the buffer must hold. */
+size_t lr_ladder_step_profile(void* device_buffer, int first_slot);
 
 /* Tuning hook, no counterpart in the reference: force the GEMV launch configuration
  * (rows-per-wave * 100 + K-split * 10 + unroll; 0 restores the built-in shape heuristic).

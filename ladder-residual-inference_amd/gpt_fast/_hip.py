@@ -38,6 +38,7 @@ _PROTOS = {
                                       c_void_p, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "lr_ladder_step_fail_offset": (c_size_t, []),
     "lr_ladder_step_tune": (None, [c_int]),
+    "lr_ladder_step_profile": (c_size_t, [c_void_p, c_int]),
 }
 
 
