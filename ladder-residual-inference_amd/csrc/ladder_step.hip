@@ -3,73 +3,66 @@
 // Why: at batch 1 a step streams 17 GB of weights through ~720 small dependent ops.  Launched
 // one by one (even from a hipGraph) the ops pay a launch boundary each and the latency-bound
 // ones (norms, RoPE, attention, combine) cost as much as the weight streaming.  Here one
-// workgroup per CU (512 lanes = 8 waves) stays resident for the whole step and walks the layers;
-// the workgroups synchronise through event counters built from relaxed agent-scope atomics (a
-// 16-group arrival tree where latency matters: ~1.5 us on 256 CUs; acquire/release fences are
-// avoided because they write back and invalidate the whole L2).
+// workgroup per CU (512 lanes = 8 waves) stays resident for the whole step and walks the layers.
 //
 // The ladder schedule is what makes this wide: attention block t reads the residual stream
 // WITHOUT the MLP output of layer t-1 (in the reference that output is still inside an
 // all-reduce), so attention(t) and mlp(t-1) are independent and run side by side.  A "slot" t is,
 // per workgroup,
-//     join:  wait until a(t-1) and m(t-2) are complete                      [tree event, exposed]
-//     residual adds + both RMSNorms (redundantly in every workgroup)
-//     wqkv(t) rows                                  -> signal E_qkv
-//     attention workgroups (a handful): wait E_qkv, attention(t) over their key range with K/V
-//         held in registers, partial results       -> signal E_att
-//     all other workgroups: w1(t-1) rows + SwiGLU   -> signal E_act    (18 us of streaming that
-//         hides the attention latency chain)
-//     wait E_att (long since signalled), merge the partial results, wo(t) rows
-//     wait E_act (signalled a few us earlier), w2(t-1) rows               -> signal "slot done"
-// so one exposed device-wide wait per layer instead of 9 kernel launches.
+//     residual adds + both RMSNorms (redundantly in every workgroup; the residual stream itself
+//         never leaves the workgroup's LDS)
+//     wqkv(t) rows
+//     attention workgroups (a handful): attention(t) over their key range with K/V held in
+//         registers, un-normalised partial results
+//     all other workgroups: w1(t-1) rows + SwiGLU  (18 us of streaming that hides the attention
+//         latency chain)
+//     merge the partial results, wo(t) rows
+//     w2(t-1) rows
 //
-// Weight streaming does not stop at these edges: every wave walks its GEMV work as a sequence of
-// "units" (16 rows x 1 KiB of one K-slice) and always has the NEXT unit's loads in flight while it
-// multiplies the current one -- also when the next unit belongs to the next GEMV or sits behind a
-// wait (the loads are issued before the wait), so HBM stays busy through reductions, epilogues,
-// norms and synchronisation latency.
+// No barriers, flags or fences: everything that crosses workgroups (module outputs a / m, qkv,
+// activations, attention partials, argmax candidates) is exchanged as self-validating 32-bit
+// words -- 16 payload bits plus the 16-bit tag of the slot that produced them -- written and read
+// with buffer instructions carrying the sc1 (agent-coherent) policy, which bypass the
+// non-coherent per-XCD L2 lines.  A consumer optimistically loads what it needs and retries the
+// words whose tag is not yet the expected one, so a value is consumed the moment it lands and a
+// producer never waits.  Overwriting a word is safe once every workgroup has finished reading its
+// previous value; that is implied by data flow (nobody can produce slot t+1's qkv before slot
+// t's partials existed, ...) except for a / m / partials, for which every workgroup publishes a
+// "done" word after its residual bookkeeping and the attention workgroups -- through which all
+// later writes of the slot depend -- check all of them while they wait for q anyway.
+// The values stored are bf16-representable, i.e. rounded exactly where the eager reference
+// rounds (fp32 attention partials take two words).  Weights, KV cache and logits use ordinary
+// accesses (read-only, or produced for the next launch).
 //
-// Data that crosses workgroups inside the step (residual, partial sums, qkv, attention output,
-// activations) lives in a small fp32 workspace and is only touched with buffer loads/stores
-// carrying the sc1 (agent-coherent) policy bit, which bypass the non-coherent per-XCD L2 lines;
-// the values stored are bf16-representable, i.e. rounded exactly where the eager reference
-// rounds.  Weights, KV cache and logits use ordinary accesses (read-only, or produced for the
-// next launch).  GEMV rows are dealt to workgroups round-robin so that the CUs working at the
-// same time read neighbouring rows (HBM-channel friendly); inside a workgroup the waves split K,
-// partial sums meet in LDS in a fixed order -- no float atomics, bit-reproducible.
+// Weight streaming never stops at these edges: every wave walks its GEMV work of the whole slot
+// (and the first job of the next one) as a sequence of "units" (8 rows x 1 KiB of one K-slice)
+// through a prefetch cursor that runs two units ahead of the multiplier, across job boundaries,
+// reductions, epilogues, norms and waits, so each wave keeps 16 KiB of loads in flight.  GEMV
+// rows are dealt to workgroups round-robin so that the CUs working at the same time read
+// neighbouring rows (HBM-channel friendly); inside a workgroup the waves split K, partial sums
+// meet in LDS in a fixed order -- no float atomics, bit-reproducible.
 //
-// Every spin is bounded: on time-out a workgroup raises ctrl->fail and leaves; the others see the
-// flag (or time out themselves), so the grid always drains.
+// Every retry loop is bounded: on time-out a workgroup raises ctrl->fail and goes on with
+// whatever it has; everybody leaves at the end of the slot in which they see the flag, so the
+// grid always drains.
 #include "lr_common.h"
 
 namespace {
 
 constexpr int NT = 512;           // lanes per workgroup
 constexpr int NW = NT / 64;       // waves per workgroup
-constexpr int EV_GROUPS = 16;     // arrival-tree fan-in
 constexpr int NJMAX = 64;         // GEMV rows a workgroup reduces per LDS round
 constexpr int RB = 8;             // rows per unit (loads a wave issues together)
-constexpr unsigned SPIN_LIMIT = 1u << 21;
+constexpr unsigned SPIN_LIMIT = 1u << 18;
 constexpr int ATT_NI = 9;         // key iterations an attention wave keeps in registers
 constexpr int NA_MAX = 16;        // attention workgroups (partial results merged by everyone)
 constexpr int PROF_SLOTS = 4, PROF_POINTS = 12;
 constexpr int AUX_SC1 = 16;       // buffer cache policy: agent scope
 
-// A tree event: every participant arrives once per epoch; the last one raises the group flags.
-struct TreeEv {
-  unsigned root, _p0[31];
-  unsigned gcount[EV_GROUPS][32];
-  unsigned gflag[EV_GROUPS][32];
-};
-
-struct Ctrl {  // every hot word on its own 128-byte line
-  TreeEv qkv;   // wqkv(t) rows of all workgroups are stored
-  TreeEv slot;  // slot finished (a(t) and m(t-1) stored); also the closing barrier of the head
-  unsigned att_count, _p2[31];  // flat arrival counters (waited on late, latency not critical)
-  unsigned act_count, _p3[31];
-  unsigned base_qkv, base_slot, base_att, base_act, _p4[28];  // epochs / arrivals consumed by earlier steps
-  unsigned fail, _p5[31];
-  unsigned nwg, _p6[31];
+struct Ctrl {
+  unsigned epoch_base, _p0[31];  // slots consumed by earlier steps (tags continue from here)
+  unsigned fail, _p1[31];
+  unsigned nwg, _p2[31];
 };
 
 struct LayerPtrs {
@@ -91,7 +84,7 @@ struct StepParams {
   int hist_len, pos0, advance;
   unsigned char* ws;  // workspace base (Ctrl at offset 0)
   unsigned ws_bytes;
-  unsigned oR, oa, om, oqkv, oact, oopart, omlpart, ocand;  // exchange buffers, offsets in floats
+  unsigned oa, om, oqkv, oact, oopart, omlpart, ocand, odone;  // exchange buffers, offsets in 32-bit words
   unsigned long long* prof;  // optional [nwg][PROF_SLOTS][PROF_POINTS] wall-clock stamps (100 MHz)
   int prof_t0;
 };
@@ -99,35 +92,14 @@ struct StepParams {
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
 
-// ---- coherent (cross-workgroup) accesses: one buffer resource over the workspace, sc1 policy.
-//      Ordinary (non-atomic) instructions, so a lane can have several in flight.
-struct Coh {
-  __amdgpu_buffer_rsrc_t r;
-  __device__ __forceinline__ float ld(unsigned fo) const {
-    return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, fo * 4, 0, AUX_SC1));
-  }
-  __device__ __forceinline__ void ld2(unsigned fo, float& a, float& b) const {  // fo % 2 == 0
-    const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(r, fo * 4, 0, AUX_SC1);
-    a = __uint_as_float(v.x);
-    b = __uint_as_float(v.y);
-  }
-  __device__ __forceinline__ void st(unsigned fo, float v) const {
-    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), r, fo * 4, 0, AUX_SC1);
-  }
-  __device__ __forceinline__ void ld8(unsigned fo, float* f) const {  // fo % 4 == 0
-    const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(r, fo * 4, 0, AUX_SC1);
-    const u32x4_t b = __builtin_amdgcn_raw_buffer_load_b128(r, fo * 4 + 16, 0, AUX_SC1);
-    f[0] = __uint_as_float(a.x); f[1] = __uint_as_float(a.y); f[2] = __uint_as_float(a.z); f[3] = __uint_as_float(a.w);
-    f[4] = __uint_as_float(b.x); f[5] = __uint_as_float(b.y); f[6] = __uint_as_float(b.z); f[7] = __uint_as_float(b.w);
-  }
-  __device__ __forceinline__ void st8(unsigned fo, const float* f) const {
-    u32x4_t a, b;
-    a.x = __float_as_uint(f[0]); a.y = __float_as_uint(f[1]); a.z = __float_as_uint(f[2]); a.w = __float_as_uint(f[3]);
-    b.x = __float_as_uint(f[4]); b.y = __float_as_uint(f[5]); b.z = __float_as_uint(f[6]); b.w = __float_as_uint(f[7]);
-    __builtin_amdgcn_raw_buffer_store_b128(a, r, fo * 4, 0, AUX_SC1);
-    __builtin_amdgcn_raw_buffer_store_b128(b, r, fo * 4 + 16, 0, AUX_SC1);
-  }
-};
+// The lane index as a value the optimiser cannot see through: index arithmetic derived from it
+// stays inside the phase that uses it instead of being hoisted out of the layer loop (where it
+// would be kept alive, and spilled, for the whole kernel).
+__device__ __forceinline__ int opaque_tid() {
+  int t = threadIdx.x;
+  asm volatile("" : "+v"(t));
+  return t;
+}
 
 __device__ __forceinline__ unsigned cldu(const unsigned* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -135,65 +107,127 @@ __device__ __forceinline__ unsigned cldu(const unsigned* p) {
 __device__ __forceinline__ void cstu(unsigned* p, unsigned v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ unsigned cadd(unsigned* p) {
-  return __hip_atomic_fetch_add(p, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 
-// All lanes: wait for this lane's outstanding memory operations, then meet.  After it, every
-// coherent store issued by the workgroup has been acknowledged.
-__device__ __forceinline__ void drain_and_sync() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-  __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();
-}
+// ------------------------------------------------------------------------------------------------
+// Self-validating exchange words.  Every 32-bit word a workgroup hands to the others carries 16
+// payload bits (high half) and the 16-bit tag of the slot that produced it (low half, never 0).
+// A bf16-representable value is one word; an fp32 value is two.  Readers load with the sc1 policy
+// (bypassing the non-coherent L2) and simply retry until the tag is the one they expect: no flag,
+// no fence, no wait on the producer side.  A dword store is indivisible, so a word is either the
+// old slot's or the new one's.  Retries are bounded.
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ unsigned tag_of(unsigned epoch) { return epoch % 65535u + 1u; }
 
-// ---- tree event: signal (all workgroups, once per epoch) / wait.  Loads may be put in flight
-//      between the two.  `epoch` values are consumed in order and never reused.
-__device__ __forceinline__ void tree_signal(TreeEv* e, unsigned epoch) {
-  drain_and_sync();
-  if (threadIdx.x == 0) {
-    const unsigned nwg = gridDim.x;
-    const unsigned ngr = nwg < EV_GROUPS ? nwg : EV_GROUPS;
-    const unsigned g = blockIdx.x % ngr;
-    const unsigned gn = nwg / ngr + (g < nwg % ngr ? 1u : 0u);
-    if (cadd(&e->gcount[g][0]) + 1u == epoch * gn) {
-      if (cadd(&e->root) + 1u == epoch * ngr) {
-        for (unsigned i = 0; i < ngr; ++i) cstu(&e->gflag[i][0], epoch);
-      }
-    }
+struct Coh {
+  __amdgpu_buffer_rsrc_t r;
+  unsigned* fail;
+
+  __device__ __forceinline__ void st(unsigned wo, float v, unsigned tag) const {  // v is bf16-representable
+    __builtin_amdgcn_raw_buffer_store_b32((__float_as_uint(v) & 0xffff0000u) | tag, r, wo * 4, 0, AUX_SC1);
   }
-}
-
-// Bounded spin of lane 0 until *word has reached `target` (wrap-safe); the whole workgroup learns
-// the outcome.  Returns false if the step must be abandoned.
-__device__ __forceinline__ bool spin_until(const unsigned* word, unsigned target, unsigned* fail, int* s_flag) {
-  if (threadIdx.x == 0) {
-    int ok = 1;
+  __device__ __forceinline__ void st8(unsigned wo, const float* f, unsigned tag) const {  // wo % 4 == 0
+    u32x4_t a, b;
+    a.x = (__float_as_uint(f[0]) & 0xffff0000u) | tag; a.y = (__float_as_uint(f[1]) & 0xffff0000u) | tag;
+    a.z = (__float_as_uint(f[2]) & 0xffff0000u) | tag; a.w = (__float_as_uint(f[3]) & 0xffff0000u) | tag;
+    b.x = (__float_as_uint(f[4]) & 0xffff0000u) | tag; b.y = (__float_as_uint(f[5]) & 0xffff0000u) | tag;
+    b.z = (__float_as_uint(f[6]) & 0xffff0000u) | tag; b.w = (__float_as_uint(f[7]) & 0xffff0000u) | tag;
+    __builtin_amdgcn_raw_buffer_store_b128(a, r, wo * 4, 0, AUX_SC1);
+    __builtin_amdgcn_raw_buffer_store_b128(b, r, wo * 4 + 16, 0, AUX_SC1);
+  }
+  // fp32 value as two words at wo, wo + 1 (wo % 2 == 0)
+  __device__ __forceinline__ void st_f32(unsigned wo, float v, unsigned tag) const {
+    const unsigned bits = __float_as_uint(v);
+    u32x2_t w;
+    w.x = (bits & 0xffff0000u) | tag;
+    w.y = (bits << 16) | tag;
+    __builtin_amdgcn_raw_buffer_store_b64(w, r, wo * 4, 0, AUX_SC1);
+  }
+  __device__ __forceinline__ bool give_up(unsigned& spins) const {
+    if ((++spins & 255u) == 0 && (spins > SPIN_LIMIT || cldu(fail))) {
+      cstu(fail, 1u);
+      return true;
+    }
+    return false;
+  }
+  // 4 tagged words -> raw words (tags still inside); spins until all four carry `tag`
+  __device__ __forceinline__ u32x4_t poll4(unsigned wo, unsigned tag) const {
     unsigned spins = 0;
-    while ((int)(cldu(word) - target) < 0) {
-      if ((++spins & 1023u) == 0 && (spins > SPIN_LIMIT || cldu(fail))) {
-        cstu(fail, 1u);
-        ok = 0;
-        break;
-      }
-      __builtin_amdgcn_s_sleep(1);
+    for (;;) {
+      const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(r, wo * 4, 0, AUX_SC1);
+      if ((((a.x ^ tag) | (a.y ^ tag) | (a.z ^ tag) | (a.w ^ tag)) & 0xffffu) == 0) return a;
+      if (give_up(spins)) return a;
+      __builtin_amdgcn_s_sleep(2);
     }
-    s_flag[0] = ok;
   }
-  __syncthreads();
-  return s_flag[0] != 0;
+  __device__ __forceinline__ u32x2_t poll2(unsigned wo, unsigned tag) const {
+    unsigned spins = 0;
+    for (;;) {
+      const u32x2_t a = __builtin_amdgcn_raw_buffer_load_b64(r, wo * 4, 0, AUX_SC1);
+      if ((((a.x ^ tag) | (a.y ^ tag)) & 0xffffu) == 0) return a;
+      if (give_up(spins)) return a;
+      __builtin_amdgcn_s_sleep(2);
+    }
+  }
+  __device__ __forceinline__ unsigned poll1(unsigned wo, unsigned tag) const {
+    unsigned spins = 0;
+    for (;;) {
+      const unsigned a = __builtin_amdgcn_raw_buffer_load_b32(r, wo * 4, 0, AUX_SC1);
+      if (((a ^ tag) & 0xffffu) == 0) return a;
+      if (give_up(spins)) return a;
+      __builtin_amdgcn_s_sleep(2);
+    }
+  }
+  // Optimistic form: raw4/raw2 issue the load (many can be in flight), settle4/settle2 accept the
+  // words if their tags match and fall back to polling otherwise.
+  __device__ __forceinline__ u32x4_t raw4(unsigned wo) const {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, wo * 4, 0, AUX_SC1);
+  }
+  __device__ __forceinline__ unsigned raw1(unsigned wo) const {
+    return __builtin_amdgcn_raw_buffer_load_b32(r, wo * 4, 0, AUX_SC1);
+  }
+  __device__ __forceinline__ u32x2_t raw2(unsigned wo) const {
+    return __builtin_amdgcn_raw_buffer_load_b64(r, wo * 4, 0, AUX_SC1);
+  }
+  __device__ __forceinline__ u32x4_t settle4(unsigned wo, unsigned tag, const u32x4_t& a) const {
+    if ((((a.x ^ tag) | (a.y ^ tag) | (a.z ^ tag) | (a.w ^ tag)) & 0xffffu) == 0) return a;
+    return poll4(wo, tag);
+  }
+  __device__ __forceinline__ u32x2_t settle2(unsigned wo, unsigned tag, const u32x2_t& a) const {
+    if ((((a.x ^ tag) | (a.y ^ tag)) & 0xffffu) == 0) return a;
+    return poll2(wo, tag);
+  }
+  // 8 bf16-valued words -> 8 floats
+  __device__ __forceinline__ void ld8(unsigned wo, unsigned tag, float* f) const {
+    unsigned spins = 0;
+    for (;;) {
+      const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(r, wo * 4, 0, AUX_SC1);
+      const u32x4_t b = __builtin_amdgcn_raw_buffer_load_b128(r, wo * 4 + 16, 0, AUX_SC1);
+      const unsigned bad = ((a.x ^ tag) | (a.y ^ tag) | (a.z ^ tag) | (a.w ^ tag) | (b.x ^ tag) | (b.y ^ tag) |
+                            (b.z ^ tag) | (b.w ^ tag)) & 0xffffu;
+      if (bad == 0 || give_up(spins)) {
+        f[0] = __uint_as_float(a.x & 0xffff0000u); f[1] = __uint_as_float(a.y & 0xffff0000u);
+        f[2] = __uint_as_float(a.z & 0xffff0000u); f[3] = __uint_as_float(a.w & 0xffff0000u);
+        f[4] = __uint_as_float(b.x & 0xffff0000u); f[5] = __uint_as_float(b.y & 0xffff0000u);
+        f[6] = __uint_as_float(b.z & 0xffff0000u); f[7] = __uint_as_float(b.w & 0xffff0000u);
+        return;
+      }
+      __builtin_amdgcn_s_sleep(2);
+    }
+  }
+  __device__ __forceinline__ void ld2(unsigned wo, unsigned tag, float& x0, float& x1) const {
+    const u32x2_t a = poll2(wo, tag);
+    x0 = __uint_as_float(a.x & 0xffff0000u);
+    x1 = __uint_as_float(a.y & 0xffff0000u);
+  }
+};
+__device__ __forceinline__ void bf4_from(const u32x4_t& a, float* f) {
+  f[0] = __uint_as_float(a.x & 0xffff0000u); f[1] = __uint_as_float(a.y & 0xffff0000u);
+  f[2] = __uint_as_float(a.z & 0xffff0000u); f[3] = __uint_as_float(a.w & 0xffff0000u);
 }
-
-__device__ __forceinline__ bool tree_wait(TreeEv* e, unsigned epoch, unsigned* fail, int* s_flag) {
-  const unsigned nwg = gridDim.x;
-  const unsigned ngr = nwg < EV_GROUPS ? nwg : EV_GROUPS;
-  return spin_until(&e->gflag[blockIdx.x % ngr][0], epoch, fail, s_flag);
-}
-
-// flat event: arrivals only add (no return value needed, nobody stalls on it)
-__device__ __forceinline__ void flat_signal(unsigned* counter) {
-  drain_and_sync();
-  if (threadIdx.x == 0) (void)cadd(counter);
+// two fp32 values from 4 words (hi, lo, hi, lo)
+__device__ __forceinline__ void f32x2_from(const u32x4_t& a, float& v0, float& v1) {
+  v0 = __uint_as_float((a.x & 0xffff0000u) | (a.y >> 16));
+  v1 = __uint_as_float((a.z & 0xffff0000u) | (a.w >> 16));
 }
 
 // ---- per-lane accumulators -> wave totals.  reduce8: afterwards lane 16*r holds sum(v[2r]) in z0
@@ -268,6 +302,28 @@ __device__ __forceinline__ Job make_job(const u16* W, int K, int row_base, int n
   return j;
 }
 
+// The jobs of slot t, built where they are needed (few are alive at a time: they live in scalar
+// registers).  kind: 0 wqkv(t), 1 w1(t-1), 2 wo(t), 3 w2(t-1), 4 lm_head; a slot without that
+// module gets a job that owns no rows.  w1 is dealt to the workgroups that do not run attention
+// in the slot.
+__device__ __forceinline__ Job slot_job(const StepParams& p, int kind, int t, int qdim, int w, int nwg, int wave) {
+  const bool a = t < p.L, b = t >= 1 && t <= p.L;
+  if (kind == 0 && a) return make_job(p.layers[t].wqkv, p.D, 0, p.nqkv, 0, 1, w, nwg, wave);
+  if (kind == 1 && b)
+    return a ? make_job(p.layers[t - 1].w1, p.D, 0, p.I, p.I, 2, w - p.NA, nwg - p.NA, wave)
+             : make_job(p.layers[t - 1].w1, p.D, 0, p.I, p.I, 2, w, nwg, wave);
+  if (kind == 2 && a) return make_job(p.layers[t].wo, qdim, 0, p.D, 0, 1, w, nwg, wave);
+  if (kind == 3 && b) return make_job(p.layers[t - 1].w2, p.I, 0, p.D, 0, 1, w, nwg, wave);
+  if (kind == 4) return make_job(p.out_w, p.D, 0, p.V, 0, 1, w, nwg, wave);
+  return make_job(nullptr, 512, 0, 0, 0, 1, 0, 1, wave);
+}
+// first job of slot t + 1
+__device__ __forceinline__ Job next_slot_job(const StepParams& p, int t, int qdim, int w, int nwg, int wave) {
+  if (t + 1 < p.L) return slot_job(p, 0, t + 1, qdim, w, nwg, wave);
+  if (t + 1 == p.L) return slot_job(p, 1, t + 1, qdim, w, nwg, wave);
+  return slot_job(p, 4, t + 1, qdim, w, nwg, wave);
+}
+
 struct Unit {
   uint4 r[RB];
 };
@@ -304,9 +360,9 @@ enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_LOGITS = 2 };
 // reduction and epilogue.
 template <int M, int EPI>
 __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, const Job& job, const Job& next,
-                                        Unit& cur, const u16* x, float* part, unsigned out_fo, int ldo, float* cand_v,
-                                        int* cand_i, float* best_v, int* best_i) {
-  const int tid = threadIdx.x, lane = tid & 63;
+                                        Unit& cur, const u16* x, float* part, unsigned out_wo, int ldo, unsigned tag,
+                                        float* cand_v, int* cand_i, float* best_v, int* best_i) {
+  const int tid = opaque_tid(), lane = tid & 63;
   const int RPI = job.rpi;
   if (!job.active) first_unit(next, lane, cur);
   for (int j0 = 0; j0 < job.nj; j0 += NJMAX) {
@@ -379,8 +435,8 @@ __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, con
       }
       const int it = job.w + job.nwg * ((j0 / RPI) + jl);
       if (m < p.B) {
-        if (EPI == EPI_STORE) coh.st(out_fo + (unsigned)(m * ldo + it), s0);
-        if (EPI == EPI_SWIGLU) coh.st(out_fo + (unsigned)(m * ldo + it), swiglu_bf(s0, s1));
+        if (EPI == EPI_STORE) coh.st(out_wo + (unsigned)(m * ldo + it), s0, tag);
+        if (EPI == EPI_SWIGLU) coh.st(out_wo + (unsigned)(m * ldo + it), swiglu_bf(s0, s1), tag);
         if (EPI == EPI_LOGITS) p.logits[(int64_t)m * p.ldl + it] = f_to_bf(s0);
       }
       if (EPI == EPI_LOGITS) {
@@ -402,47 +458,70 @@ __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, con
 }
 
 // ------------------------------------------------------------------------------------------------
-// Residual bookkeeping + RMSNorm for the coming jobs, done redundantly by every workgroup:
-//   v1 = src (+ d1);  v2 = v1 (+ d2);  each add rounded to bf16.
-//   x1 = norm(v1) * g1 -> LDS (if g1);  x2 = norm(v2) * g2 -> LDS (if g2);  workgroup 0 stores v2.
-// src is either the coherent fp32 residual or rows of the bf16 embedding table.
+// Residual bookkeeping + RMSNorm for the coming jobs, done redundantly by every workgroup (each
+// keeps its own copy of the residual stream in LDS, so only module outputs are ever exchanged):
+//   v1 = R (+ d1);  v2 = v1 (+ d2);  each add rounded to bf16;  R <- v2.
+//   x1 = norm(v1) * g1 -> LDS (if g1);  x2 = norm(v2) * g2 -> LDS (if g2).
+// At the first slot R comes from rows of the bf16 embedding table.  d1/d2 are tagged exchange
+// arrays; all their loads are issued before the first one is checked.
 // ------------------------------------------------------------------------------------------------
+constexpr int PRO_NIT = 4;  // 8-element chunks per lane and row: dim <= PRO_NIT * NT * 8
+
 template <int M>
-__device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, unsigned src_fo, const int* emb_rows,
-                                         bool has_d1, unsigned d1_fo, bool has_d2, unsigned d2_fo, const u16* g1,
-                                         const u16* g2, bool write_r, unsigned rout_fo, u16* x1, u16* x2, float* red) {
-  const int tid = threadIdx.x, D = p.D;
+__device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, u16* xr, const int* emb_rows,
+                                         bool has_d1, unsigned d1_wo, unsigned d1_tag, bool has_d2, unsigned d2_wo,
+                                         unsigned d2_tag, const u16* g1, const u16* g2, u16* x1, u16* x2, float* red) {
+  const int tid = opaque_tid(), D = p.D;
   float ss1[M], ss2[M];
   // pass 1: the (bf16-exact) sums go to LDS unscaled; sums of squares per lane
 #pragma unroll
   for (int m = 0; m < M; ++m) {
     ss1[m] = ss2[m] = 0.0f;
-    for (int c = tid * 8; c < D; c += NT * 8) {
-      float v[8], t1[8], t2[8];
-      if (emb_rows) {
-        const int id = emb_rows[m];
-        const bool ok = id >= 0 && id < p.vocab;
-        unpack8(ok ? ld16(p.tok_emb + (int64_t)id * D + c) : make_uint4(0, 0, 0, 0), v);
-      } else {
-        coh.ld8(src_fo + m * D + c, v);
+    u32x4_t r1[PRO_NIT][2], r2[PRO_NIT][2];
+#pragma unroll
+    for (int it = 0; it < PRO_NIT; ++it) {
+      const int c = (it * NT + tid) * 8;
+      if (c < D && has_d1) {
+        r1[it][0] = coh.raw4(d1_wo + m * D + c);
+        r1[it][1] = coh.raw4(d1_wo + m * D + c + 4);
       }
-      if (has_d1) coh.ld8(d1_fo + m * D + c, t1);
-      if (has_d2) coh.ld8(d2_fo + m * D + c, t2);
-      if (has_d1) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = round_bf(v[j] + t1[j]);
+      if (c < D && has_d2) {
+        r2[it][0] = coh.raw4(d2_wo + m * D + c);
+        r2[it][1] = coh.raw4(d2_wo + m * D + c + 4);
       }
-      if (g1) st16(x1 + m * D + c, pack8(v));
+    }
 #pragma unroll
-      for (int j = 0; j < 8; ++j) ss1[m] += v[j] * v[j];
-      if (has_d2) {
+    for (int it = 0; it < PRO_NIT; ++it) {
+      const int c = (it * NT + tid) * 8;
+      if (c < D) {
+        float v[8], t[8];
+        if (emb_rows) {
+          const int id = emb_rows[m];
+          const bool ok = id >= 0 && id < p.vocab;
+          unpack8(ok ? ld16(p.tok_emb + (int64_t)id * D + c) : make_uint4(0, 0, 0, 0), v);
+        } else {
+          unpack8(*reinterpret_cast<const uint4*>(xr + m * D + c), v);
+        }
+        if (has_d1) {
+          bf4_from(coh.settle4(d1_wo + m * D + c, d1_tag, r1[it][0]), t);
+          bf4_from(coh.settle4(d1_wo + m * D + c + 4, d1_tag, r1[it][1]), t + 4);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = round_bf(v[j] + t2[j]);
+          for (int j = 0; j < 8; ++j) v[j] = round_bf(v[j] + t[j]);
+        }
+        if (g1) st16(x1 + m * D + c, pack8(v));
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss1[m] += v[j] * v[j];
+        if (has_d2) {
+          bf4_from(coh.settle4(d2_wo + m * D + c, d2_tag, r2[it][0]), t);
+          bf4_from(coh.settle4(d2_wo + m * D + c + 4, d2_tag, r2[it][1]), t + 4);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) v[j] = round_bf(v[j] + t[j]);
+        }
+        if (g2) st16(x2 + m * D + c, pack8(v));
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss2[m] += v[j] * v[j];
+        st16(xr + m * D + c, pack8(v));
       }
-      if (g2) st16(x2 + m * D + c, pack8(v));
-#pragma unroll
-      for (int j = 0; j < 8; ++j) ss2[m] += v[j] * v[j];
-      if (write_r && blockIdx.x == 0) coh.st8(rout_fo + m * D + c, v);
     }
   }
 #pragma unroll
@@ -489,12 +568,13 @@ __device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, un
   __syncthreads();
 }
 
-// Bring a coherent fp32 activation [M][K] (bf16-representable values) into LDS as bf16.
+// Bring a tagged activation [M][K] into LDS as bf16 (waits for every word).
 template <int M>
-__device__ __forceinline__ void load_x(const Coh& coh, unsigned src_fo, int K, u16* x) {
-  for (int c = threadIdx.x * 8; c < M * K; c += NT * 8) {
+__device__ __forceinline__ void load_x(const Coh& coh, unsigned src_wo, unsigned tag, int K, u16* x) {
+  const int tid_ = opaque_tid();
+  for (int c = tid_ * 8; c < M * K; c += NT * 8) {
     float f[8];
-    coh.ld8(src_fo + c, f);
+    coh.ld8(src_wo + c, tag, f);
     st16(x + c, pack8(f));
   }
   __syncthreads();
@@ -503,9 +583,9 @@ __device__ __forceinline__ void load_x(const Coh& coh, unsigned src_fo, int K, u
 // ------------------------------------------------------------------------------------------------
 // Attention of slot t in attention workgroup `aw` of NA: keys [k0, k1) of every (sequence, kv
 // head), all G q heads of the kv head at once so K and V are read once per GQA group.  The K and V
-// rows of the key range are loaded into registers in one go (before the wait for qkv), scores,
+// rows of the key range are loaded into registers in one go (before q is waited for), scores,
 // softmax and P.V stay in fp32; each workgroup publishes an un-normalised partial result with its
-// own (max, sum).
+// own (max, sum) as tagged fp32 word pairs.
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ void rope_pair(float x0, float x1, float c, float s, float& o0, float& o1) {
 #pragma clang fp contract(off)
@@ -514,16 +594,16 @@ __device__ __forceinline__ void rope_pair(float x0, float x1, float c, float s, 
   o1 = round_bf(d + e);
 }
 
-template <int HD>
 struct KV {
   uint4 k[ATT_NI], v[ATT_NI];
 };
 
 template <int HD>
 __device__ __forceinline__ void attention_load(const StepParams& p, const LayerPtrs& lp, int b, int kvh, int k0,
-                                               int k1, int pos, KV<HD>& kv) {
+                                               int k1, int pos, KV& kv) {
   constexpr int LPK = HD / 8, KPW = 64 / LPK;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int tid_ = opaque_tid();
+  const int wave = tid_ >> 6, lane = tid_ & 63;
   const int kl = lane / LPK, dl = (lane % LPK) * 8;
   const u16* kbase = lp.k_cache + ((int64_t)b * p.Hkv + kvh) * p.Smax * HD;
   const u16* vbase = lp.v_cache + ((int64_t)b * p.Hkv + kvh) * p.Smax * HD;
@@ -543,11 +623,13 @@ __device__ __forceinline__ void attention_load(const StepParams& p, const LayerP
 
 template <int M, int HD, int G>
 __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh& coh, const LayerPtrs& lp, int b,
-                                                  int kvh, int k0, int k1, int pos, KV<HD>& kv, float* qs, float* sc,
-                                                  int sc_ld, float* ored, float* knew, float* vnew, float* s_m,
-                                                  float* s_l) {
+                                                  int kvh, int k0, int k1, int pos, unsigned tag, bool poll_done,
+                                                  unsigned long long* stamp,
+                                                  KV& kv, float* qs,
+                                                  float* sc, int sc_ld, float* ored, float* knew, float* vnew,
+                                                  float* s_m, float* s_l) {
   constexpr int LPK = HD / 8, KPW = 64 / LPK;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = opaque_tid(), wave = tid >> 6, lane = tid & 63;
   const int aw = blockIdx.x, NA = p.NA, Hkv = p.Hkv, Hq = Hkv * G;
   const int n = k1 - k0;
   const bool owner = pos >= k0 && pos < k1;
@@ -555,23 +637,45 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
   const u16* trow = p.rope + (int64_t)pos * HD;  // (cos, sin) pairs of this position
   const int kl = lane / LPK, dl = (lane % LPK) * 8;
   const unsigned qkv = p.oqkv + (unsigned)(b * p.nqkv);
-  const unsigned o_out = p.oopart + (unsigned)((((b * Hq + kvh * G) * NA) + aw) * HD);
-  const unsigned ml_out = p.omlpart + (unsigned)((((b * Hq + kvh * G) * NA) + aw) * 2);
+  // partial outputs: [b * Hq + h][NA][HD] fp32 as word pairs; (max, sum): [b * Hq + h][NA] as 4 words
+  const unsigned o_out = p.oopart + (unsigned)((((b * Hq + kvh * G) * NA) + aw) * HD * 2);
+  const unsigned ml_out = p.omlpart + (unsigned)((((b * Hq + kvh * G) * NA) + aw) * 4);
 
+  // ---- every workgroup has finished reading the previous slot's exchange data once its "done"
+  //      word carries this slot's tag: only then may partial results (and, downstream of them,
+  //      module outputs) be overwritten
+  // Everything this phase waits for is requested at once; what has not landed yet is polled.
+  const bool own = owner && tid < HD / 2;
+  const unsigned ko = qkv + (unsigned)(Hq * HD + kvh * HD + 2 * tid), vo = ko + (unsigned)(Hkv * HD);
+  const unsigned q0 = qkv + (unsigned)(kvh * G * HD + 2 * tid);  // pair `tid` of the G * HD / 2 pairs of this group
+  unsigned dr = 0;
+  u32x2_t qr = {0u, 0u}, rk = {0u, 0u}, rv = {0u, 0u};
+  if (poll_done && tid < (int)gridDim.x) dr = coh.raw1(p.odone + (unsigned)tid);
+  if (tid < G * HD / 2) qr = coh.raw2(q0);
+  if (own) {
+    rk = coh.raw2(ko);
+    rv = coh.raw2(vo);
+  }
+  if (poll_done) {
+    if (tid < (int)gridDim.x && ((dr ^ tag) & 0xffffu) != 0) coh.poll1(p.odone + (unsigned)tid, tag);
+    for (int i = tid + NT; i < (int)gridDim.x; i += NT) coh.poll1(p.odone + (unsigned)i, tag);
+  }
   // ---- rotate q (all G heads) into LDS; the owner of `pos` also rotates k, keeps k/v in LDS and
   //      writes them to the cache for the following steps
   for (int i = tid; i < G * HD / 2; i += NT) {
     const int g = i / (HD / 2), j = i - g * (HD / 2);
-    float x0, x1;
-    coh.ld2(qkv + (unsigned)((kvh * G + g) * HD + 2 * j), x0, x1);
+    const unsigned qo = qkv + (unsigned)((kvh * G + g) * HD + 2 * j);
+    const u32x2_t sq = i == tid ? coh.settle2(qo, tag, qr) : coh.poll2(qo, tag);
     const u32 cs = *reinterpret_cast<const u32*>(trow + 2 * j);
-    rope_pair(x0, x1, bf_lo(cs), bf_hi(cs), qs[g * HD + 2 * j], qs[g * HD + 2 * j + 1]);
+    rope_pair(__uint_as_float(sq.x & 0xffff0000u), __uint_as_float(sq.y & 0xffff0000u), bf_lo(cs), bf_hi(cs),
+              qs[g * HD + 2 * j], qs[g * HD + 2 * j + 1]);
   }
-  if (owner && tid < HD / 2) {
+  if (own) {
     const int j = tid;
-    float kx0, kx1, v0, v1, r0, r1;
-    coh.ld2(qkv + (unsigned)(Hq * HD + kvh * HD + 2 * j), kx0, kx1);
-    coh.ld2(qkv + (unsigned)((Hq + Hkv) * HD + kvh * HD + 2 * j), v0, v1);
+    const u32x2_t sk = coh.settle2(ko, tag, rk), sv = coh.settle2(vo, tag, rv);
+    const float kx0 = __uint_as_float(sk.x & 0xffff0000u), kx1 = __uint_as_float(sk.y & 0xffff0000u);
+    const float v0 = __uint_as_float(sv.x & 0xffff0000u), v1 = __uint_as_float(sv.y & 0xffff0000u);
+    float r0, r1;
     const u32 cs = *reinterpret_cast<const u32*>(trow + 2 * j);
     rope_pair(kx0, kx1, bf_lo(cs), bf_hi(cs), r0, r1);
     knew[2 * j] = r0; knew[2 * j + 1] = r1;
@@ -581,42 +685,40 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
     *reinterpret_cast<u32*>(lp.v_cache + slot) = pack_bf2(v0, v1);
   }
   __syncthreads();
+  if (stamp && tid == 0) stamp[8] = wall_clock64();
   if (n <= 0) {
-    for (int i = tid; i < G * HD; i += NT) coh.st(o_out + (unsigned)((i / HD) * NA * HD + (i % HD)), 0.0f);
+    for (int i = tid; i < G * HD; i += NT)
+      coh.st_f32(o_out + (unsigned)(((i / HD) * NA * HD + (i % HD)) * 2), 0.0f, tag);
     if (tid < G) {
-      coh.st(ml_out + (unsigned)(tid * NA * 2), -INFINITY);
-      coh.st(ml_out + (unsigned)(tid * NA * 2 + 1), 0.0f);
+      coh.st_f32(ml_out + (unsigned)(tid * NA * 4), -INFINITY, tag);
+      coh.st_f32(ml_out + (unsigned)(tid * NA * 4 + 2), 0.0f, tag);
     }
     __syncthreads();
     return;
   }
   // ---- scores
-  {
-    float qf[G][8];
 #pragma unroll
-    for (int g = 0; g < G; ++g)
+  for (int i = 0; i < ATT_NI; ++i) {
+    const int key = k0 + (i * NW + wave) * KPW + kl;
+    float kf[8];
+    unpack8(kv.k[i], kf);
+    if (key == pos) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) qf[g][j] = qs[g * HD + dl + j];
+      for (int j = 0; j < 8; ++j) kf[j] = knew[dl + j];
+    }
 #pragma unroll
-    for (int i = 0; i < ATT_NI; ++i) {
-      const int key = k0 + (i * NW + wave) * KPW + kl;
-      float kf[8];
-      unpack8(kv.k[i], kf);
-      if (key == pos) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) kf[j] = knew[dl + j];
-      }
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-        float s = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) s = fmaf(kf[j], qf[g][j], s);
-        s = LPK == 16 ? row_sum16(s) : half_row_sum8(s);
-        if (key < k1 && (lane % LPK) == 0) sc[g * sc_ld + key - k0] = s * scale;
-      }
+    for (int g = 0; g < G; ++g) {
+      const float4 qa = *reinterpret_cast<const float4*>(qs + g * HD + dl);
+      const float4 qb = *reinterpret_cast<const float4*>(qs + g * HD + dl + 4);
+      float s = kf[0] * qa.x;
+      s = fmaf(kf[1], qa.y, s); s = fmaf(kf[2], qa.z, s); s = fmaf(kf[3], qa.w, s);
+      s = fmaf(kf[4], qb.x, s); s = fmaf(kf[5], qb.y, s); s = fmaf(kf[6], qb.z, s); s = fmaf(kf[7], qb.w, s);
+      s = LPK == 16 ? row_sum16(s) : half_row_sum8(s);
+      if (key < k1 && (lane % LPK) == 0) sc[g * sc_ld + key - k0] = s * scale;
     }
   }
   __syncthreads();
+  if (stamp && tid == 0) stamp[9] = wall_clock64();
   // ---- softmax statistics: a wave per head; sc becomes exp(s - max)
   for (int g = wave; g < G; g += NW) {
     float m = -INFINITY;
@@ -632,65 +734,50 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
     if (lane == 0) { s_m[g] = m; s_l[g] = l; }
   }
   __syncthreads();
-  // ---- P.V, folded over the key groups of a wave, then over the waves in two LDS rounds
-  float acc[G][8];
+  if (stamp && tid == 0) stamp[10] = wall_clock64();
+  // ---- P.V: head by head, folded over the key groups of a wave, then over the waves in LDS
+#pragma unroll 2
+  for (int g = 0; g < G; ++g) {
+    float acc[8];
 #pragma unroll
-  for (int g = 0; g < G; ++g)
+    for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[g][j] = 0.0f;
+    for (int i = 0; i < ATT_NI; ++i) {
+      const int key = k0 + (i * NW + wave) * KPW + kl;
+      if (key < k1) {
+        float vf[8];
+        unpack8(kv.v[i], vf);
+        if (key == pos) {
 #pragma unroll
-  for (int i = 0; i < ATT_NI; ++i) {
-    const int key = k0 + (i * NW + wave) * KPW + kl;
-    if (key < k1) {
-      float vf[8];
-      unpack8(kv.v[i], vf);
-      if (key == pos) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) vf[j] = vnew[dl + j];
-      }
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
+          for (int j = 0; j < 8; ++j) vf[j] = vnew[dl + j];
+        }
         const float pr = sc[g * sc_ld + key - k0];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[g][j] = fmaf(pr, vf[j], acc[g][j]);
+        for (int j = 0; j < 8; ++j) acc[j] = fmaf(pr, vf[j], acc[j]);
       }
     }
-  }
-#pragma unroll
-  for (int g = 0; g < G; ++g)
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      float v = acc[g][j];
+      float v = acc[j];
 #pragma unroll
       for (int o = LPK; o < 64; o <<= 1) v += __shfl_xor(v, o, LR_WAVE);
-      acc[g][j] = v;
+      acc[j] = v;
     }
-  if (wave >= NW / 2 && kl == 0) {
-#pragma unroll
-    for (int g = 0; g < G; ++g)
-#pragma unroll
-      for (int j = 0; j < 8; ++j) ored[((wave - NW / 2) * G + g) * HD + dl + j] = acc[g][j];
-  }
-  __syncthreads();
-  if (wave < NW / 2 && kl == 0) {
-#pragma unroll
-    for (int g = 0; g < G; ++g)
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        float* slot = &ored[(wave * G + g) * HD + dl + j];
-        *slot = acc[g][j] + *slot;
-      }
+    if (kl == 0) {
+      *reinterpret_cast<float4*>(ored + (wave * G + g) * HD + dl) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+      *reinterpret_cast<float4*>(ored + (wave * G + g) * HD + dl + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
+    }
   }
   __syncthreads();
   for (int i = tid; i < G * HD; i += NT) {
     float v = 0.0f;
 #pragma unroll
-    for (int wv = 0; wv < NW / 2; ++wv) v += ored[wv * G * HD + i];
-    coh.st(o_out + (unsigned)((i / HD) * NA * HD + (i % HD)), v);
+    for (int wv = 0; wv < NW; ++wv) v += ored[wv * G * HD + i];
+    coh.st_f32(o_out + (unsigned)(((i / HD) * NA * HD + (i % HD)) * 2), v, tag);
   }
   if (tid < G) {
-    coh.st(ml_out + (unsigned)(tid * NA * 2), s_m[tid]);
-    coh.st(ml_out + (unsigned)(tid * NA * 2 + 1), s_l[tid]);
+    coh.st_f32(ml_out + (unsigned)(tid * NA * 4), s_m[tid], tag);
+    coh.st_f32(ml_out + (unsigned)(tid * NA * 4 + 2), s_l[tid], tag);
   }
   __syncthreads();
 }
@@ -698,50 +785,39 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
 // Every workgroup: merge the NA partial attention results into y [M][Hq * HD] (bf16, LDS).
 //   y = sum_s w_s o_s,  w_s = exp(m_s - max) / sum_s' exp(m_s' - max) l_s'
 template <int M, int HD>
-__device__ __forceinline__ void attention_merge(const StepParams& p, const Coh& coh, int Hq, u16* y, float* wbuf) {
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+__device__ __forceinline__ void attention_merge(const StepParams& p, const Coh& coh, int Hq, unsigned tag, u16* y,
+                                                float* wbuf) {
+  const int tid = opaque_tid(), wave = tid >> 6, lane = tid & 63;
   const int NA = p.NA, nbh = p.B * Hq;
   const int npairs = nbh * HD / 2;
-  float o0[NA_MAX], o1[NA_MAX];
-  // the first batch of partial outputs goes in flight together with the (max, sum) pairs
-  int pp = tid;
-  if (pp < npairs) {
-    const int bh = (2 * pp) / HD, d = (2 * pp) % HD;
-#pragma unroll
-    for (int s = 0; s < NA_MAX; ++s) {
-      o0[s] = o1[s] = 0.0f;
-      if (s < NA) coh.ld2(p.oopart + (unsigned)((bh * NA + s) * HD + d), o0[s], o1[s]);
-    }
-  }
   // weights: a wave per (sequence, head); lanes < NA hold one chunk each
   for (int bh = wave; bh < nbh; bh += NW) {
     float m = -INFINITY, l = 0.0f;
-    if (lane < NA) coh.ld2(p.omlpart + (unsigned)((bh * NA + lane) * 2), m, l);
+    if (lane < NA) f32x2_from(coh.poll4(p.omlpart + (unsigned)((bh * NA + lane) * 4), tag), m, l);
     const float mx = wave_max(m);
     const float w = m == -INFINITY ? 0.0f : expf(m - mx);
     const float L = wave_sum(w * l);
     if (lane < NA) wbuf[bh * NA_MAX + lane] = L > 0.0f ? w / L : 0.0f;
   }
   __syncthreads();
-  while (pp < npairs) {
-    const int bh = (2 * pp) / HD;
+  for (int pp = tid; pp < npairs; pp += NT) {
+    const int bh = (2 * pp) / HD, d = (2 * pp) % HD;
     float y0 = 0.0f, y1 = 0.0f;
+    u32x4_t raw[NA_MAX];
+#pragma unroll
+    for (int s = 0; s < NA_MAX; ++s)
+      if (s < NA) raw[s] = coh.raw4(p.oopart + (unsigned)(((bh * NA + s) * HD + d) * 2));
 #pragma unroll
     for (int s = 0; s < NA_MAX; ++s) {
       if (s < NA) {
+        float o0, o1;
+        f32x2_from(coh.settle4(p.oopart + (unsigned)(((bh * NA + s) * HD + d) * 2), tag, raw[s]), o0, o1);
         const float w = wbuf[bh * NA_MAX + s];
-        y0 = fmaf(w, o0[s], y0);
-        y1 = fmaf(w, o1[s], y1);
+        y0 = fmaf(w, o0, y0);
+        y1 = fmaf(w, o1, y1);
       }
     }
     *reinterpret_cast<u32*>(y + 2 * pp) = pack_bf2(y0, y1);
-    pp += NT;
-    if (pp < npairs) {
-      const int bh2 = (2 * pp) / HD, d2 = (2 * pp) % HD;
-#pragma unroll
-      for (int s = 0; s < NA_MAX; ++s)
-        if (s < NA) coh.ld2(p.oopart + (unsigned)((bh2 * NA + s) * HD + d2), o0[s], o1[s]);
-    }
   }
   __syncthreads();
 }
@@ -755,13 +831,14 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   const int xlen = M * (D > I ? D : I);
   const int sc_ld = ATT_NI * NW * (64 / (HD / 8));      // keys an attention workgroup can hold
   u16* xa = reinterpret_cast<u16*>(smem);              // attention-chain input  [M][<= D]
-  u16* xb = xa + xlen;                                  // MLP-chain input        [M][<= D]
-  float* part = reinterpret_cast<float*>(xb + xlen);    // [NW][NJMAX * M]
+  u16* xb = xa + xlen;                                  // MLP-chain input        [M][<= max(D, I)]
+  u16* xr = xb + xlen;                                  // residual stream        [M][D]
+  float* part = reinterpret_cast<float*>(xr + M * D);   // [NW][NJMAX * M]
   float* red = part + NW * NJMAX * M;                   // [NW][M][2]
   float* qs = red + NW * M * 2;                         // [G][HD]
   float* sc = qs + G * HD;                              // [G][sc_ld]
-  float* ored = sc + G * sc_ld;                         // [NW/2][G][HD]
-  float* knew = ored + (NW / 2) * G * HD;               // [HD]
+  float* ored = sc + G * sc_ld;                         // [NW][G][HD]
+  float* knew = ored + NW * G * HD;                     // [HD]
   float* vnew = knew + HD;                              // [HD]
   float* s_m = vnew + HD;                               // [G]
   float* s_l = s_m + G;                                 // [G]
@@ -776,16 +853,10 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   Ctrl* ctrl = reinterpret_cast<Ctrl*>(p.ws);
   Coh coh;
   coh.r = __builtin_amdgcn_make_buffer_rsrc(p.ws, 0, (int)p.ws_bytes, 0x00020000);
-  if (tid == 0) {
-    s_flag[1] = (int)cldu(&ctrl->base_qkv);
-    s_flag[2] = (int)cldu(&ctrl->base_slot);
-    s_flag[3] = (int)cldu(&ctrl->base_att);
-    s_flag[4] = (int)cldu(&ctrl->base_act);
-  }
+  coh.fail = &ctrl->fail;
+  if (tid == 0) s_flag[1] = (int)cldu(&ctrl->epoch_base);
   __syncthreads();
-  const unsigned base_qkv = (unsigned)s_flag[1], base_slot = (unsigned)s_flag[2];
-  const unsigned base_att = (unsigned)s_flag[3], base_act = (unsigned)s_flag[4];
-  __syncthreads();
+  const unsigned epoch_base = (unsigned)s_flag[1];
   int pos = p.pos[0];
   pos = pos < 0 ? 0 : (pos >= p.Smax ? p.Smax - 1 : pos);
   const bool att_wg = w < NA;
@@ -795,131 +866,145 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   const int k0 = w * chunk;
   const int k1 = k0 + chunk < nkeys ? k0 + chunk : nkeys;
 
-  const Job none = make_job(nullptr, 512, 0, 0, 0, 1, 0, 1, wave);
+  const int qdim = Hq * HD;
   Unit cur;
-  first_unit(make_job(p.layers[0].wqkv, D, 0, p.nqkv, 0, 1, w, nwg, wave), lane, cur);
+  first_unit(slot_job(p, 0, 0, qdim, w, nwg, wave), lane, cur);
 
 #define LR_STAMP(k)                                                                                  \
   if (p.prof && t >= p.prof_t0 && t < p.prof_t0 + PROF_SLOTS && tid == 0)                            \
     p.prof[((size_t)blockIdx.x * PROF_SLOTS + (t - p.prof_t0)) * PROF_POINTS + (k)] = wall_clock64();
+#define LR_JOB(kind) slot_job(p, kind, t, qdim, w, nwg, wave)
   for (int t = 0; t <= L; ++t) {
     const bool has_a = t < L, has_b = t >= 1;
-    const LayerPtrs la = p.layers[has_a ? t : L - 1];
-    const LayerPtrs lb = p.layers[has_b ? t - 1 : 0];
-    // jobs of this slot in execution order (absent ones own no rows).  w1 is dealt to the
-    // workgroups that do not run attention in this slot.
-    const Job j_qkv = has_a ? make_job(la.wqkv, D, 0, p.nqkv, 0, 1, w, nwg, wave) : none;
-    const Job j_w1 = !has_b ? none
-                            : (has_a ? make_job(lb.w1, D, 0, I, I, 2, w - NA, nwg - NA, wave)
-                                     : make_job(lb.w1, D, 0, I, I, 2, w, nwg, wave));
-    const Job j_wo = has_a ? make_job(la.wo, Hq * HD, 0, D, 0, 1, w, nwg, wave) : none;
-    const Job j_w2 = has_b ? make_job(lb.w2, I, 0, D, 0, 1, w, nwg, wave) : none;
-    const Job j_nxt = t + 1 < L ? make_job(p.layers[t + 1].wqkv, D, 0, p.nqkv, 0, 1, w, nwg, wave)
-                                : (t + 1 == L ? make_job(p.layers[L - 1].w1, D, 0, I, I, 2, w, nwg, wave)
-                                              : make_job(p.out_w, D, 0, p.V, 0, 1, w, nwg, wave));
+    const LayerPtrs* la = p.layers + (has_a ? t : L - 1);
+    const LayerPtrs* lb = p.layers + (has_b ? t - 1 : 0);
+    const unsigned tag = tag_of(epoch_base + (unsigned)t + 1u), tag_prev = tag_of(epoch_base + (unsigned)t);
+    const unsigned act_wo = p.oact + (unsigned)((t & 1) * M * I);  // activations alternate between two buffers
     LR_STAMP(0)
     // ---------------- v1 = R + m(t-2) feeds mlp(t-1); v2 = v1 + a(t-1) feeds attention(t)
-    prologue<M>(p, coh, p.oR + (unsigned)(((t + 1) & 1) * M * D), t == 0 ? p.tokens : nullptr, t >= 2, p.om,
-                t >= 1 && has_a, p.oa, has_b ? lb.ffn_norm : nullptr, has_a ? la.attn_norm : nullptr, true,
-                p.oR + (unsigned)((t & 1) * M * D), xb, xa, red);
+    prologue<M>(p, coh, xr, t == 0 ? p.tokens : nullptr, t >= 2, p.om, tag_prev, t >= 1 && has_a, p.oa, tag_prev,
+                has_b ? lb->ffn_norm : nullptr, has_a ? la->attn_norm : nullptr, xb, xa, red);
+    // this workgroup no longer reads a / m / the previous partials
+    if (tid == 0) coh.st(p.odone + (unsigned)w, 0.0f, tag);
     LR_STAMP(1)
-    run_job<M, EPI_STORE>(p, coh, j_qkv, j_w1, cur, xa, part, p.oqkv, p.nqkv, nullptr, nullptr, nullptr, nullptr);
-    LR_STAMP(2)
-    if (has_a) tree_signal(&ctrl->qkv, base_qkv + (unsigned)t + 1u);
     if (has_a && att_wg) {
-      // ---------------- attention workgroup: K/V of (sequence 0, head 0) go in flight, then wait for qkv
-      KV<HD> kv;
-      attention_load<HD>(p, la, 0, 0, k0, k1, pos, kv);
-      if (!tree_wait(&ctrl->qkv, base_qkv + (unsigned)t + 1u, &ctrl->fail, s_flag)) return;
-      LR_STAMP(3)
+      run_job<M, EPI_STORE>(p, coh, LR_JOB(0), LR_JOB(2), cur, xa, part, p.oqkv, p.nqkv, tag, nullptr, nullptr,
+                            nullptr, nullptr);
+      LR_STAMP(2)
+      // ---------------- attention workgroup (it owns no rows of w1)
+      KV kv;
+      bool first = true;
       for (int b = 0; b < p.B; ++b)
         for (int kvh = 0; kvh < p.Hkv; ++kvh) {
-          if (b + kvh > 0) attention_load<HD>(p, la, b, kvh, k0, k1, pos, kv);
-          attention_compute<M, HD, G>(p, coh, la, b, kvh, k0, k1, pos, kv, qs, sc, sc_ld, ored, knew, vnew, s_m, s_l);
+          attention_load<HD>(p, *la, b, kvh, k0, k1, pos, kv);
+          attention_compute<M, HD, G>(p, coh, *la, b, kvh, k0, k1, pos, tag, first,
+                                      (p.prof && t >= p.prof_t0 && t < p.prof_t0 + PROF_SLOTS)
+                                          ? p.prof + ((size_t)blockIdx.x * PROF_SLOTS + (t - p.prof_t0)) * PROF_POINTS
+                                          : nullptr,
+                                      kv, qs, sc, sc_ld, ored, knew, vnew, s_m, s_l);
+          first = false;
         }
-      flat_signal(&ctrl->att_count);
-      first_unit(j_wo, lane, cur);
-      LR_STAMP(4)
     } else {
+      run_job<M, EPI_STORE>(p, coh, LR_JOB(0), LR_JOB(1), cur, xa, part, p.oqkv, p.nqkv, tag, nullptr, nullptr,
+                            nullptr, nullptr);
+      LR_STAMP(2)
       // ---------------- everyone else: the up/gate projection of the previous layer + SwiGLU
-      LR_STAMP(3)
-      run_job<M, EPI_SWIGLU>(p, coh, j_w1, has_a ? j_wo : j_w2, cur, xb, part, p.oact, I, nullptr, nullptr, nullptr,
-                             nullptr);
-      LR_STAMP(4)
+      run_job<M, EPI_SWIGLU>(p, coh, LR_JOB(1), has_a ? LR_JOB(2) : LR_JOB(3), cur, xb, part, act_wo, I, tag, nullptr,
+                             nullptr, nullptr, nullptr);
     }
-    if (has_b) flat_signal(&ctrl->act_count);
-    LR_STAMP(5)
+    LR_STAMP(3)
     // ---------------- merge attention partials, output projection
     if (has_a) {
-      if (!spin_until(&ctrl->att_count, base_att + (unsigned)(t + 1) * (unsigned)NA, &ctrl->fail, s_flag)) return;
-      LR_STAMP(6)
-      attention_merge<M, HD>(p, coh, Hq, xa, wbuf);
-      LR_STAMP(7)
-      run_job<M, EPI_STORE>(p, coh, j_wo, j_w2, cur, xa, part, p.oa, D, nullptr, nullptr, nullptr, nullptr);
+      attention_merge<M, HD>(p, coh, Hq, tag, xa, wbuf);
+      LR_STAMP(4)
+      run_job<M, EPI_STORE>(p, coh, LR_JOB(2), has_b ? LR_JOB(3) : next_slot_job(p, t, qdim, w, nwg, wave), cur, xa,
+                            part, p.oa, D, tag, nullptr, nullptr, nullptr, nullptr);
+    } else if (has_b) {
+      // no attention in this slot, hence nobody has checked the "done" words yet: do it here,
+      // before the down projection overwrites m
+      for (int i = tid; i < nwg; i += NT) coh.poll1(p.odone + (unsigned)i, tag);
     }
-    LR_STAMP(8)
+    LR_STAMP(5)
     // ---------------- down projection of the previous layer
     if (has_b) {
-      if (!spin_until(&ctrl->act_count, base_act + (unsigned)t * (unsigned)nwg, &ctrl->fail, s_flag)) return;
-      load_x<M>(coh, p.oact, I, xb);
-      run_job<M, EPI_STORE>(p, coh, j_w2, none, cur, xb, part, p.om, D, nullptr, nullptr, nullptr, nullptr);
+      load_x<M>(coh, act_wo, tag, I, xb);
+      LR_STAMP(6)
+      run_job<M, EPI_STORE>(p, coh, LR_JOB(3), next_slot_job(p, t, qdim, w, nwg, wave), cur, xb, part, p.om, D, tag,
+                            nullptr, nullptr, nullptr, nullptr);
     }
-    LR_STAMP(9)
-    tree_signal(&ctrl->slot, base_slot + (unsigned)t + 1u);
-    first_unit(j_nxt, lane, cur);  // next slot's first weights, in flight across the join
-    if (!tree_wait(&ctrl->slot, base_slot + (unsigned)t + 1u, &ctrl->fail, s_flag)) return;
-    LR_STAMP(10)
+    LR_STAMP(7)
+    // one workgroup-wide look at the failure flag per slot keeps a broken step from running on
+    if (tid == 0) s_flag[0] = (int)cldu(&ctrl->fail);
+    __syncthreads();
+    if (s_flag[0]) return;
   }
+#undef LR_JOB
 #undef LR_STAMP
-  // ---------------- head: x = (R + a) + m, final norm, vocab-shard lm_head, argmax
-  prologue<M>(p, coh, p.oR + (unsigned)((L & 1) * M * D), nullptr, true, p.oa, true, p.om, nullptr, p.final_norm,
-              false, 0u, xb, xa, red);
+  // ---------------- head: x = (R + a(L-1)) + m(L-1), final norm, vocab-shard lm_head, argmax
+  const unsigned tag = tag_of(epoch_base + (unsigned)L + 2u), tag_prev = tag_of(epoch_base + (unsigned)L + 1u);
+  prologue<M>(p, coh, xr, nullptr, true, p.oa, tag_of(epoch_base + (unsigned)L), true, p.om, tag_prev, nullptr,
+              p.final_norm, xb, xa, red);
   float best_v = -INFINITY;
   int best_i = 0x7fffffff;
-  run_job<M, EPI_LOGITS>(p, coh, make_job(p.out_w, D, 0, p.V, 0, 1, w, nwg, wave), none, cur, xa, part, 0u, 0, cand_v,
-                         cand_i, &best_v, &best_i);
-  if (tid < M) {
-    coh.st(p.ocand + (unsigned)((w * M + tid) * 2), best_v);
-    coh.st(p.ocand + (unsigned)((w * M + tid) * 2 + 1), __int_as_float(best_i));
+  run_job<M, EPI_LOGITS>(p, coh, slot_job(p, 4, L + 1, qdim, w, nwg, wave), slot_job(p, -1, 0, qdim, w, nwg, wave), cur,
+                         xa, part, 0u, 0, tag,
+                         cand_v, cand_i, &best_v, &best_i);
+  if (tid < M) {  // candidate: value (bf16-exact), a filler word, index as two 16-bit halves
+    const unsigned wo = p.ocand + (unsigned)((w * M + tid) * 4);
+    coh.st(wo, best_v, tag);
+    coh.st(wo + 1, 0.0f, tag);
+    coh.st_f32(wo + 2, __int_as_float(best_i), tag);
   }
-  tree_signal(&ctrl->slot, base_slot + (unsigned)L + 2u);
-  if (!tree_wait(&ctrl->slot, base_slot + (unsigned)L + 2u, &ctrl->fail, s_flag)) return;
   if (w == 0) {
-    if (tid < p.B) {
+    for (int m = 0; m < p.B; ++m) {
       float bv = -INFINITY;
       int bi = 0x7fffffff;
-      for (int wg = 0; wg < nwg; ++wg) {
-        float v, fi;
-        coh.ld2(p.ocand + (unsigned)((wg * M + tid) * 2), v, fi);
-        const int i = __float_as_int(fi);
+      for (int wg = tid; wg < nwg; wg += NT) {
+        const u32x4_t c = coh.poll4(p.ocand + (unsigned)((wg * M + m) * 4), tag);
+        const float v = __uint_as_float(c.x & 0xffff0000u);
+        const int i = (int)((c.z & 0xffff0000u) | (c.w >> 16));
         if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
       }
-      if (bi == 0x7fffffff) bi = 0;
-      if (p.next_token) p.next_token[tid] = bi;
-      if (p.advance && p.cur_token) p.cur_token[tid] = bi;
-      const int slot = p.pos[0] - p.pos0;
-      if (p.advance && p.history && slot >= 0 && slot < p.hist_len) p.history[(int64_t)tid * p.ld_hist + slot] = bi;
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, LR_WAVE);
+        const int oi = __shfl_xor(bi, o, LR_WAVE);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+      }
+      __syncthreads();
+      if (lane == 0) { cand_v[wave] = bv; cand_i[wave] = bi; }
+      __syncthreads();
+      if (tid == 0) {
+        for (int wv = 1; wv < NW; ++wv)
+          if (cand_v[wv] > bv || (cand_v[wv] == bv && cand_i[wv] < bi)) { bv = cand_v[wv]; bi = cand_i[wv]; }
+        if (bi == 0x7fffffff) bi = 0;
+        if (p.next_token) p.next_token[m] = bi;
+        if (p.advance && p.cur_token) p.cur_token[m] = bi;
+        const int slot = p.pos[0] - p.pos0;
+        if (p.advance && p.history && slot >= 0 && slot < p.hist_len) p.history[(int64_t)m * p.ld_hist + slot] = bi;
+      }
     }
     __syncthreads();
     if (tid == 0) {
       if (p.advance) p.pos[0] = p.pos[0] + 1;
-      cstu(&ctrl->base_qkv, base_qkv + (unsigned)L);
-      cstu(&ctrl->base_slot, base_slot + (unsigned)L + 2u);
-      cstu(&ctrl->base_att, base_att + (unsigned)L * (unsigned)NA);
-      cstu(&ctrl->base_act, base_act + (unsigned)L * (unsigned)nwg);
+      cstu(&ctrl->epoch_base, (epoch_base + (unsigned)L + 2u) % 65535u);
     }
   }
 }
 
-__global__ void k_step_init(Ctrl* c, unsigned nwg) {
-  unsigned* w = reinterpret_cast<unsigned*>(c);
-  for (int i = threadIdx.x; i < (int)(sizeof(Ctrl) / 4); i += blockDim.x) w[i] = 0u;
-  __syncthreads();
-  if (threadIdx.x == 0) c->nwg = nwg;
+__global__ void k_step_init(Ctrl* c, unsigned nwg, unsigned* words, unsigned n_words) {
+  // control block and every exchange word start at zero: tag 0 is never a valid tag
+  unsigned* cw = reinterpret_cast<unsigned*>(c);
+  for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < n_words; i += gridDim.x * blockDim.x) words[i] = 0u;
+  if (blockIdx.x == 0) {
+    for (int i = threadIdx.x; i < (int)(sizeof(Ctrl) / 4); i += blockDim.x) cw[i] = 0u;
+    __syncthreads();
+    if (threadIdx.x == 0) c->nwg = nwg;
+  }
 }
 
 struct Layout {
-  size_t ctrl, Rbuf, abuf, mbuf, qkv, act, opart, mlpart, cand, total;
+  size_t ctrl, abuf, mbuf, qkv, act, opart, mlpart, cand, done, total;
 };
 
 static int num_cus() {
@@ -955,14 +1040,14 @@ static Layout make_layout(const lr_ladder_model_t* md, int B, int nwg) {
   Layout l;
   size_t o = 0;
   l.ctrl = o; o = up(o + sizeof(Ctrl));
-  l.Rbuf = o; o = up(o + sizeof(float) * 2 * B * D);
-  l.abuf = o; o = up(o + sizeof(float) * B * D);
-  l.mbuf = o; o = up(o + sizeof(float) * B * D);
-  l.qkv = o; o = up(o + sizeof(float) * B * nqkv);
-  l.act = o; o = up(o + sizeof(float) * B * md->ffn);
-  l.opart = o; o = up(o + sizeof(float) * B * Hq * na * hd);
-  l.mlpart = o; o = up(o + sizeof(float) * B * Hq * na * 2);
-  l.cand = o; o = up(o + sizeof(float) * nwg * B * 2);
+  l.abuf = o; o = up(o + 4 * (size_t)B * D);
+  l.mbuf = o; o = up(o + 4 * (size_t)B * D);
+  l.qkv = o; o = up(o + 4 * (size_t)B * nqkv);
+  l.act = o; o = up(o + 4 * (size_t)2 * B * md->ffn);
+  l.opart = o; o = up(o + 4 * (size_t)B * Hq * na * hd * 2);
+  l.mlpart = o; o = up(o + 4 * (size_t)B * Hq * na * 4);
+  l.cand = o; o = up(o + 4 * (size_t)nwg * B * 4);
+  l.done = o; o = up(o + 4 * (size_t)nwg);
   l.total = o;
   return l;
 }
@@ -982,9 +1067,9 @@ static bool has_instance(int B, int hd, int G) {
 template <int M, int HD, int G>
 static size_t lds_bytes(int D, int I, int Hq) {
   const int xlen = M * (D > I ? D : I);
-  const size_t fl = (size_t)NW * NJMAX * M + NW * M * 2 + G * HD + (size_t)G * att_capacity(HD) + (NW / 2) * G * HD +
+  const size_t fl = (size_t)NW * NJMAX * M + NW * M * 2 + G * HD + (size_t)G * att_capacity(HD) + NW * G * HD +
                     2 * HD + 2 * G + (size_t)M * Hq * NA_MAX + 2 * NJMAX * M + 8;
-  return (size_t)xlen * 2 * sizeof(u16) + fl * sizeof(float);
+  return ((size_t)xlen * 2 + (size_t)M * D) * sizeof(u16) + fl * sizeof(float) + 16;
 }
 
 static size_t lds_need(int B, int hd, int G, int D, int I, int Hq) {
@@ -999,7 +1084,7 @@ static int validate(const lr_ladder_model_t* md, int B) {
   if (B < 1 || md->dim <= 0 || md->n_layer <= 0 || md->n_head <= 0 || md->n_kv_head <= 0 || md->ffn <= 0 ||
       md->out_rows <= 0 || md->vocab <= 0 || md->smax <= 0 || md->block_size <= 0 || md->n_head % md->n_kv_head)
     return LR_E_SHAPE;
-  if (B > 2 || md->dim > 16384 || md->dim % 8 || md->ffn % 8 || (md->head_dim != 64 && md->head_dim != 128))
+  if (B > 2 || md->dim > PRO_NIT * NT * 8 || md->dim % 8 || md->ffn % 8 || (md->head_dim != 64 && md->head_dim != 128))
     return LR_E_UNSUPPORTED;
   const int G = md->n_head / md->n_kv_head;
   if (!has_instance(B, md->head_dim, G)) return LR_E_UNSUPPORTED;
@@ -1053,9 +1138,11 @@ extern "C" int lr_ladder_step_init(const lr_ladder_model_t* md, int batch, void*
   if (rc != LR_OK) return rc;
   LR_REQUIRE_PTR(workspace);
   if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return LR_E_ALIGN;
-  if (bytes < make_layout(md, batch, num_cus()).total) return LR_E_SHAPE;
-  k_step_init<<<dim3(1), dim3(256), 0, (hipStream_t)stream>>>(reinterpret_cast<Ctrl*>(workspace),
-                                                             (unsigned)num_cus());
+  const Layout l = make_layout(md, batch, num_cus());
+  if (bytes < l.total) return LR_E_SHAPE;
+  k_step_init<<<dim3(64), dim3(256), 0, (hipStream_t)stream>>>(reinterpret_cast<Ctrl*>(workspace), (unsigned)num_cus(),
+                                                              reinterpret_cast<unsigned*>(workspace),
+                                                              (unsigned)(l.total / 4));
   return lr_launch_status();
 }
 
@@ -1087,9 +1174,10 @@ extern "C" int lr_ladder_decode_step(const lr_ladder_model_t* md, int batch, con
   sp.hist_len = hist_len; sp.pos0 = pos0; sp.advance = advance;
   sp.ws = reinterpret_cast<unsigned char*>(workspace);
   sp.ws_bytes = (unsigned)l.total;
-  sp.oR = (unsigned)(l.Rbuf / 4); sp.oa = (unsigned)(l.abuf / 4); sp.om = (unsigned)(l.mbuf / 4);
+  sp.oa = (unsigned)(l.abuf / 4); sp.om = (unsigned)(l.mbuf / 4);
   sp.oqkv = (unsigned)(l.qkv / 4); sp.oact = (unsigned)(l.act / 4);
   sp.oopart = (unsigned)(l.opart / 4); sp.omlpart = (unsigned)(l.mlpart / 4); sp.ocand = (unsigned)(l.cand / 4);
+  sp.odone = (unsigned)(l.done / 4);
   sp.prof = g_prof;
   sp.prof_t0 = g_prof_t0;
   hipStream_t s = (hipStream_t)stream;
