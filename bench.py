@@ -10,13 +10,15 @@ so the KV cache has its real length, and the timed steps start at position 2048.
 steps read is resident in HBM when the clock starts.
 
 Prints ONE JSON line.  `value` = decoded tokens per second (whole job = the one GPU).
-`roofline`   : the dominant kernel, the weight-streaming GEMV on the w1 (up+gate) projection
-               [7168 x 8192] -- 47 % of a step's bytes.  `achieved` = its algorithmic bytes per launch
-               (weight matrix + input row(s) + output row(s)) / its mean launch duration, measured
-               here with HIP events around 80 back-to-back launches over the 80 layers' distinct
-               matrices (so nothing is served from cache) on the launch stream.
-`step_roofline`: the same ratio for the whole decode step: algorithmic bytes per step (all weights
-               and gains once + valid KV + KV write + embedding rows) / measured step time.
+`roofline`   : the dominant kernel.  For the ladder model at batch <= 2 that is k_ladder_step, ONE
+               persistent launch per decode step; `achieved` = algorithmic bytes per launch (all
+               weights and gains once + valid KV + KV write + embedding rows + logits) / its mean
+               launch duration, measured here with HIP events around back-to-back launches on the
+               launch stream.  `traffic` = HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE
+               counter runs (a constant recorded from those runs, or null).  Other models / batches
+               fall back to the per-op path, whose dominant kernel is the w1 GEMV.
+`step_roofline`: the same ratio for the whole decode step as replayed from the hipGraph (kernel +
+               token hand-over): algorithmic bytes per step / measured step time.
 `cpu_baseline`: the oracle (a PyTorch-CPU restatement of the reference; the reference itself cannot
                run without CUDA + NCCL) timed on this machine's host cores on the reference's
                CPU-sized case: Ladder-1B fp32, batch 1, 128-token prompt, greedy decode."""
@@ -31,6 +33,9 @@ sys.path.insert(0, os.path.join(ROOT, "ladder-residual-inference_amd"))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes one k_ladder_step launch moves on the headline workload, from the rocprofv3 counter runs
+# summarised under profiles/ (None until measured).
+TRAFFIC_BYTES_PER_LAUNCH = 17.737e9  # B=1, prompt 2048; 1.016 x algorithmic
 
 
 def cpu_baseline(new_tokens=32, repeats=2):
@@ -71,6 +76,9 @@ def main():
     ap.add_argument("--prompt", type=int, default=2048)
     ap.add_argument("--model", type=str, default="gpt_ladder:ladder-70b-tp8")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (reads 1 GiB, writes 1 GiB) a few times: under "
+                         "rocprofv3 --pmc its FETCH_SIZE / WRITE_SIZE readings calibrate the counters' unit")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures ONE tensor-parallel rank's shard on ONE GPU (partial sums stay local, no "
@@ -104,6 +112,14 @@ def main():
     prefill_s = time.perf_counter() - t0
     dg = bm.get_cuda_graphs_for_decode(model, prompt, B, new, first, greedy=True)
 
+    if args.calibrate_copy:
+        src = torch.zeros(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     # ---- W untimed steps, then exactly K timed steps from position T
     dg.reset(first)
     for _ in range(W):
@@ -121,26 +137,48 @@ def main():
     step_bytes = sum(bm.decode_bytes_per_step(cfg, B, T + i) for i in range(K)) / K
     step_gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
 
-    # ---- dominant kernel: w1 GEMV, HIP events on the launch stream, distinct matrix per launch
-    w1s = [blk.feed_forward.w1.weight for blk in model.layers] if hasattr(model.layers[0], "feed_forward") else \
-        [blk.attention.wqkv1.weight for blk in model.layers]
-    N, Kdim = w1s[0].shape
-    x = torch.randn(B, Kdim, device=dev).to(torch.bfloat16)
-    y = torch.empty(B, N, device=dev, dtype=torch.bfloat16)
-    for w in w1s[:8]:
-        _hip.linear(x, w, y)
-    reps = 3
+    # ---- dominant kernel, timed with HIP events on the stream it is launched on (torch's current stream)
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    ev0.record()
-    for _ in range(reps):
-        for w in w1s:
+    fused = getattr(model, "use_fused_step", False) and hasattr(model, "decode_step_fused") and \
+        model._fused_step(B) is not None
+    if fused:
+        # the whole step is ONE kernel (k_ladder_step): algorithmic bytes per launch = bytes per step
+        pos = torch.tensor([T], dtype=torch.int32, device=dev)
+        tok = first.view(B, 1).to(torch.int32).contiguous()
+        for _ in range(3):
+            model.decode_step_fused(tok, pos)
+        reps = 30
+        torch.cuda.synchronize()
+        ev0.record()
+        for _ in range(reps):
+            model.decode_step_fused(tok, pos)
+        ev1.record()
+        torch.cuda.synchronize()
+        k_us = 1e3 * ev0.elapsed_time(ev1) / reps
+        k_bytes = bm.decode_bytes_per_step(cfg, B, T)
+        k_name = (f"k_ladder_step (one persistent launch = the whole decode step at position {T}: "
+                  f"{cfg.n_layer} layers + lm_head, M={B})")
+    else:
+        # per-op path: the weight-streaming GEMV on the w1 (up+gate) projection, a distinct matrix per launch
+        w1s = [blk.feed_forward.w1.weight for blk in model.layers] if hasattr(model.layers[0], "feed_forward") else \
+            [blk.attention.wqkv1.weight for blk in model.layers]
+        N, Kdim = w1s[0].shape
+        x = torch.randn(B, Kdim, device=dev).to(torch.bfloat16)
+        y = torch.empty(B, N, device=dev, dtype=torch.bfloat16)
+        for w in w1s[:8]:
             _hip.linear(x, w, y)
-    ev1.record()
-    torch.cuda.synchronize()
-    gemv_us = 1e3 * ev0.elapsed_time(ev1) / (reps * len(w1s))
-    gemv_bytes = 2 * (N * Kdim + B * Kdim + B * N)
-    gemv_gbps = gemv_bytes / (gemv_us * 1e-6) / 1e9
+        reps = 3
+        torch.cuda.synchronize()
+        ev0.record()
+        for _ in range(reps):
+            for w in w1s:
+                _hip.linear(x, w, y)
+        ev1.record()
+        torch.cuda.synchronize()
+        k_us = 1e3 * ev0.elapsed_time(ev1) / (reps * len(w1s))
+        k_bytes = 2 * (N * Kdim + B * Kdim + B * N)
+        k_name = f"k_gemv (w1 up+gate projection, [{N} x {Kdim}] bf16, M={B})"
+    k_gbps = k_bytes / (k_us * 1e-6) / 1e9
 
     out = {
         "metric": "decode_tokens_per_sec", "value": round(B * 1e3 / ms_per_step, 2), "unit": "tok/s",
@@ -152,10 +190,10 @@ def main():
                    "batch": B, "prompt_len": T, "virtual_tp": cfg.tp_world_size},
         "ms_per_token": round(ms_per_step, 4),
         "prefill_s": round(prefill_s, 4),
-        "roofline": {"bound": "hbm", "kernel": f"k_gemv (w1 up+gate projection, [{N} x {Kdim}] bf16, M={B})",
-                     "achieved": round(gemv_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gemv_gbps / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "bytes_per_launch": gemv_bytes, "avg_launch_us": round(gemv_us, 3)},
+        "roofline": {"bound": "hbm", "kernel": k_name,
+                     "achieved": round(k_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(k_gbps / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH if fused else None,
+                     "bytes_per_launch": int(k_bytes), "avg_launch_us": round(k_us, 3)},
         "step_roofline": {"bound": "hbm", "achieved": round(step_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                           "frac": round(step_gbps / HBM_PEAK_GBPS, 4), "bytes_per_step": int(step_bytes)},
         "first_tokens": tokens,

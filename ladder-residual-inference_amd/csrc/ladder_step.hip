@@ -52,7 +52,7 @@ namespace {
 constexpr int NT = 512;           // lanes per workgroup
 constexpr int NW = NT / 64;       // waves per workgroup
 constexpr int NJMAX = 64;         // GEMV rows a workgroup reduces per LDS round
-constexpr int RB = 8;             // rows per unit (loads a wave issues together)
+constexpr int RB = 8;  // rows per unit (loads a wave issues together)
 constexpr unsigned SPIN_LIMIT = 1u << 18;
 constexpr int ATT_NI = 9;         // key iterations an attention wave keeps in registers
 constexpr int NA_MAX = 16;        // attention workgroups (partial results merged by everyone)
