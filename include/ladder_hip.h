@@ -158,10 +158,11 @@ int lr_ladder_step_init(const lr_ladder_model_t* model, int batch, void* workspa
  *     history[b, pos[0] - pos0] = next_token[b] (if history),  cur_token[b] = next_token[b] (if
  *     cur_token),  pos[0] += 1,
  * so that replaying the captured step is a complete decode loop.  tokens and cur_token may alias.
- * The kernel occupies every CU and synchronises them with device-wide barriers: nothing else may
- * run on the device concurrently, and two steps must not overlap.  Barrier waits are bounded; if
- * one ever expires the workspace word at lr_ladder_step_fail_offset() becomes non-zero, the
- * outputs of that step are undefined and the workspace must be initialised again. */
+ * The kernel occupies every CU (one resident workgroup each) and the workgroups wait for each
+ * other's results: nothing else may run on the device concurrently, and two steps must not
+ * overlap.  Every wait is bounded; if one ever expires the workspace word at
+ * lr_ladder_step_fail_offset() becomes non-zero, the outputs of that step are undefined and the
+ * workspace must be initialised again. */
 int lr_ladder_decode_step(const lr_ladder_model_t* model, int batch, const int32_t* tokens, int32_t* pos, void* logits,
                           int64_t ldl, int32_t* next_token, int advance, int32_t* cur_token, int32_t* history,
                           int64_t ld_hist, int hist_len, int pos0, void* workspace, size_t bytes, lr_stream_t stream);

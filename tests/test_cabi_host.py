@@ -1,0 +1,143 @@
+"""CPU-side checks of the C-ABI library and the host logic above it (no kernel is launched).
+
+* libladder_hip.so loads and exports every symbol include/ladder_hip.h declares, and the ctypes
+  prototypes of gpt_fast/_hip.py cover exactly that set;
+* argument validation answers before anything touches the device;
+* the configuration registry reproduces the reference's shapes (gpt_ladder_TP.py:20-207) and the
+  per-rank sizes of the benchmark configurations;
+* modules built on the meta device carry the reference's parameter names and shapes;
+* bytes-per-step accounting used for the roofline."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "ladder_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(lr_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from gpt_fast import _hip
+
+    if not os.path.exists(_hip.lib_path()):
+        pytest.fail(f"{_hip.lib_path()} has not been built (python ladder-residual-inference_amd/build.py)")
+    return _hip.load()
+
+
+def test_library_exports_every_declared_symbol(lib):
+    from gpt_fast import _hip
+
+    names = declared_symbols()
+    assert len(names) >= 20
+    raw = ctypes.CDLL(_hip.lib_path())
+    missing = [n for n in names if not hasattr(raw, n)]
+    assert not missing, missing
+    assert sorted(_hip.exported_names()) == names
+
+
+def test_version_and_error_strings(lib):
+    assert lib.lr_version() >= 1
+    seen = set()
+    for code in range(0, -6, -1):
+        s = lib.lr_error_string(code)
+        assert s and s.decode()
+        seen.add(s)
+    assert len(seen) >= 5, "every error code has its own message"
+
+
+def test_validation_precedes_any_device_work(lib):
+    # null / misaligned pointers and impossible shapes are refused on the host (no GPU here)
+    E_NULL, E_ALIGN, E_SHAPE = -1, -2, -3
+    assert lib.lr_add(None, None, 1.0, None, 16, None) == E_NULL
+    assert lib.lr_add(8, 16, 1.0, 32, 16, None) == E_ALIGN
+    assert lib.lr_linear(None, 0, None, None, 0, 1, 8, 8, 0, None) == E_NULL
+    assert lib.lr_linear(64, 8, 128, 256, 8, 0, 8, 8, 0, None) == E_SHAPE
+    assert lib.lr_argmax(None, 0, None, 1, 8, None) == E_NULL
+    assert lib.lr_ladder_decode_step(None, 1, None, None, None, 0, None, 0, None, None, 0, 0, 0, None, 0, None) == E_NULL
+    assert lib.lr_ladder_step_workspace_bytes(None, 1) == 0
+
+
+def test_missing_library_is_an_error(monkeypatch):
+    from gpt_fast import _hip
+
+    monkeypatch.setattr(_hip, "_lib", None)
+    monkeypatch.setattr(_hip, "_LIB_PATH", os.path.join(ROOT, "no_such_dir", "libladder_hip.so"))
+    with pytest.raises(_hip.LadderHipError):
+        _hip.load()
+
+
+def test_registry_matches_reference_shapes():
+    from gpt_fast.config import ModelArgs, args_from_name
+
+    a = args_from_name("ladder", "llama-3-8b")
+    assert (a.dim, a.n_layer, a.n_head, a.n_local_heads, a.intermediate_size, a.vocab_size) == \
+        (4096, 32, 32, 8, 14336, 128256)
+    assert a.head_dim == 128 and a.rope_base == 500000
+    # default intermediate size: round_up(int(8 * dim / 3), 256)   (gpt_ladder_TP.py:56-60)
+    b = ModelArgs(dim=1000, n_head=8, n_layer=1)
+    assert b.intermediate_size == 2816 and b.n_local_heads == 8 and b.head_dim == 125
+    # one tensor-parallel rank of Ladder-70B at TP = 8
+    c = args_from_name("ladder", "ladder-70b-tp8")
+    assert (c.tp_world_size, c.n_head_local, c.n_kv_local, c.ffn_local, c.output_rows) == (8, 8, 1, 3584, 16032)
+    d = args_from_name("ladder", "ladder-405b-tp8")
+    assert (d.dim, d.n_layer, d.n_head_local, d.n_kv_local, d.ffn_local) == (16384, 126, 16, 1, 6656)
+    with pytest.raises(AssertionError):
+        ModelArgs(dim=512, n_head=8, n_layer=1, intermediate_size=1022, tp_world_size=4)   # not divisible by tp
+    from gpt_fast.utils import Attention
+
+    with pytest.raises(AssertionError), torch.device("meta"):   # heads not divisible by tp (utils.py:155-162)
+        Attention(ModelArgs(dim=512, n_head=8, n_local_heads=2, n_layer=1, intermediate_size=1024, tp_world_size=4))
+
+
+@pytest.mark.parametrize("family", ["ladder", "dense", "desync", "parallel"])
+def test_meta_modules_have_reference_parameter_names(family):
+    import benchmark as bm
+    from gpt_fast.config import ModelArgs
+    from oracle import ladder_oracle as O
+
+    kw = dict(block_size=64, vocab_size=512, n_layer=2, n_head=4, n_local_heads=2, dim=256, intermediate_size=512)
+    cls = {"ladder": bm.GPTLadder, "dense": bm.GPTDense, "desync": bm.GPTDesync, "parallel": bm.GPTParallel}[family]
+    with torch.device("meta"):
+        model = cls(ModelArgs(**kw))
+    got = {n: tuple(p.shape) for n, p in model.named_parameters()}
+    want = dict(O.param_shapes(O.OracleConfig(**kw), family))
+    assert got == want
+
+
+def test_virtual_tp_builds_one_rank_without_a_process_group(monkeypatch):
+    from gpt_fast import maybe_init_dist, tp
+
+    assert maybe_init_dist() == 0
+    tp.set_virtual_tp(8, 3)
+    try:
+        assert tp.get_tp_world_size() == 8 and tp.get_tp_rank() == 3
+    finally:
+        tp.set_virtual_tp(1, 0)
+    with pytest.raises(AssertionError):
+        tp.set_virtual_tp(4, 4)
+    assert not torch.distributed.is_initialized()
+    monkeypatch.setenv("WORLD_SIZE", "2")     # a multi-process launch is refused, never silently run
+    with pytest.raises(RuntimeError):
+        maybe_init_dist()
+
+
+def test_bytes_per_step_accounting():
+    import benchmark as bm
+    from gpt_fast.config import args_from_name
+
+    c = args_from_name("ladder", "ladder-70b-tp8")
+    b0 = bm.decode_bytes_per_step(c, 1, 2048)
+    # weights 17.378 GB + valid KV + KV write + embedding row + logits: 17.462 GB at position 2048
+    assert abs(b0 - 17.462e9) < 0.003e9
+    # one more position costs one more K and V row per layer
+    assert bm.decode_bytes_per_step(c, 1, 2049) - b0 == 80 * 2 * 128 * 2
+    # a second sequence adds its KV, embedding row and logits, not the weights
+    assert bm.decode_bytes_per_step(c, 2, 2048) - b0 < 0.1e9
