@@ -587,6 +587,12 @@ __device__ __forceinline__ void load_x(const Coh& coh, unsigned src_wo, unsigned
 // softmax and P.V stay in fp32; each workgroup publishes an un-normalised partial result with its
 // own (max, sum) as tagged fp32 word pairs.
 // ------------------------------------------------------------------------------------------------
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+// c + a.lo * b.lo + a.hi * b.hi on packed bf16 pairs, fp32 accumulation
+__device__ __forceinline__ float dot2(u32 a, u32 b, float c) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
+}
+
 __device__ __forceinline__ void rope_pair(float x0, float x1, float c, float s, float& o0, float& o1) {
 #pragma clang fp contract(off)
   const float a = x0 * c, b = x1 * s, d = x1 * c, e = x0 * s;
@@ -625,8 +631,8 @@ template <int M, int HD, int G>
 __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh& coh, const LayerPtrs& lp, int b,
                                                   int kvh, int k0, int k1, int pos, unsigned tag, bool poll_done,
                                                   unsigned long long* stamp,
-                                                  KV& kv, float* qs,
-                                                  float* sc, int sc_ld, float* ored, float* knew, float* vnew,
+                                                  KV& kv, u32* qp,
+                                                  float* sc, int sc_ld, float* ored, u32* kp, float* vnew,
                                                   float* s_m, float* s_l) {
   constexpr int LPK = HD / 8, KPW = 64 / LPK;
   const int tid = opaque_tid(), wave = tid >> 6, lane = tid & 63;
@@ -667,8 +673,9 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
     const unsigned qo = qkv + (unsigned)((kvh * G + g) * HD + 2 * j);
     const u32x2_t sq = i == tid ? coh.settle2(qo, tag, qr) : coh.poll2(qo, tag);
     const u32 cs = *reinterpret_cast<const u32*>(trow + 2 * j);
-    rope_pair(__uint_as_float(sq.x & 0xffff0000u), __uint_as_float(sq.y & 0xffff0000u), bf_lo(cs), bf_hi(cs),
-              qs[g * HD + 2 * j], qs[g * HD + 2 * j + 1]);
+    float r0, r1;
+    rope_pair(__uint_as_float(sq.x & 0xffff0000u), __uint_as_float(sq.y & 0xffff0000u), bf_lo(cs), bf_hi(cs), r0, r1);
+    qp[g * (HD / 2) + j] = pack_bf2(r0, r1);  // exact: both were just rounded to bf16
   }
   if (own) {
     const int j = tid;
@@ -678,7 +685,7 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
     float r0, r1;
     const u32 cs = *reinterpret_cast<const u32*>(trow + 2 * j);
     rope_pair(kx0, kx1, bf_lo(cs), bf_hi(cs), r0, r1);
-    knew[2 * j] = r0; knew[2 * j + 1] = r1;
+    kp[j] = pack_bf2(r0, r1);
     vnew[2 * j] = v0; vnew[2 * j + 1] = v1;
     const int64_t slot = (((int64_t)b * Hkv + kvh) * p.Smax + pos) * HD + 2 * j;
     *reinterpret_cast<u32*>(lp.k_cache + slot) = pack_bf2(r0, r1);
@@ -696,25 +703,23 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
     __syncthreads();
     return;
   }
-  // ---- scores
+  // ---- scores: K and q are bf16 pairs, so a pair of products per v_dot2_f32_bf16 (fp32 sums)
 #pragma unroll
   for (int i = 0; i < ATT_NI; ++i) {
-    const int key = k0 + (i * NW + wave) * KPW + kl;
-    float kf[8];
-    unpack8(kv.k[i], kf);
-    if (key == pos) {
+    if (i * NW * KPW < n) {  // uniform: later iterations hold no key of this range
+      const int key = k0 + (i * NW + wave) * KPW + kl;
+      uint4 kk = kv.k[i];
+      if (key == pos) kk = *reinterpret_cast<const uint4*>(kp + dl / 2);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) kf[j] = knew[dl + j];
-    }
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      const float4 qa = *reinterpret_cast<const float4*>(qs + g * HD + dl);
-      const float4 qb = *reinterpret_cast<const float4*>(qs + g * HD + dl + 4);
-      float s = kf[0] * qa.x;
-      s = fmaf(kf[1], qa.y, s); s = fmaf(kf[2], qa.z, s); s = fmaf(kf[3], qa.w, s);
-      s = fmaf(kf[4], qb.x, s); s = fmaf(kf[5], qb.y, s); s = fmaf(kf[6], qb.z, s); s = fmaf(kf[7], qb.w, s);
-      s = LPK == 16 ? row_sum16(s) : half_row_sum8(s);
-      if (key < k1 && (lane % LPK) == 0) sc[g * sc_ld + key - k0] = s * scale;
+      for (int g = 0; g < G; ++g) {
+        const uint4 q4 = *reinterpret_cast<const uint4*>(qp + g * (HD / 2) + dl / 2);
+        float s = dot2(kk.x, q4.x, 0.0f);
+        s = dot2(kk.y, q4.y, s);
+        s = dot2(kk.z, q4.z, s);
+        s = dot2(kk.w, q4.w, s);
+        s = LPK == 16 ? row_sum16(s) : half_row_sum8(s);
+        if (key < k1 && (lane % LPK) == 0) sc[g * sc_ld + key - k0] = s * scale;
+      }
     }
   }
   __syncthreads();
@@ -735,37 +740,53 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
   }
   __syncthreads();
   if (stamp && tid == 0) stamp[10] = wall_clock64();
-  // ---- P.V: head by head, folded over the key groups of a wave, then over the waves in LDS
-#pragma unroll 2
-  for (int g = 0; g < G; ++g) {
-    float acc[8];
+  // ---- P.V: GB heads at a time share the unpacked V rows; the key groups of a wave are folded with
+  //      lane-half / lane-row swaps (one swap + one add folds two accumulators), the waves in LDS
+  constexpr int GB = G < 8 ? G : 8;
+#pragma unroll 1
+  for (int g0 = 0; g0 < G; g0 += GB) {
+    float acc[GB][8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
+    for (int g = 0; g < GB; ++g)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[g][j] = 0.0f;
 #pragma unroll
     for (int i = 0; i < ATT_NI; ++i) {
-      const int key = k0 + (i * NW + wave) * KPW + kl;
-      if (key < k1) {
+      if (i * NW * KPW < n) {
+        const int key = k0 + (i * NW + wave) * KPW + kl;
         float vf[8];
         unpack8(kv.v[i], vf);
         if (key == pos) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) vf[j] = vnew[dl + j];
         }
-        const float pr = sc[g * sc_ld + key - k0];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[j] = fmaf(pr, vf[j], acc[j]);
+        for (int g = 0; g < GB; ++g) {
+          const float pr = key < k1 ? sc[(g0 + g) * sc_ld + key - k0] : 0.0f;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) acc[g][j] = fmaf(pr, vf[j], acc[g][j]);
+        }
       }
     }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      float v = acc[j];
+    for (int g = 0; g < GB; ++g) {
+      if (LPK == 8) {  // 8 key groups: fold lane bit 3 first
 #pragma unroll
-      for (int o = LPK; o < 64; o <<= 1) v += __shfl_xor(v, o, LR_WAVE);
-      acc[j] = v;
-    }
-    if (kl == 0) {
-      *reinterpret_cast<float4*>(ored + (wave * G + g) * HD + dl) = make_float4(acc[0], acc[1], acc[2], acc[3]);
-      *reinterpret_cast<float4*>(ored + (wave * G + g) * HD + dl + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
+        for (int j = 0; j < 8; ++j) acc[g][j] += dpp_mov<0x128>(acc[g][j]);  // row_ror:8
+      }
+      float w[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        swap32(acc[g][j], acc[g][j + 4]);
+        w[j] = acc[g][j] + acc[g][j + 4];
+      }
+      swap16(w[0], w[2]);
+      swap16(w[1], w[3]);
+      // lane row r = lane / 16 now holds the wave totals of elements 2r (z0) and 2r + 1 (z1) of the
+      // lane's 8-element slice
+      const float z0 = w[0] + w[2], z1 = w[1] + w[3];
+      if (LPK == 16 || (lane & 8) == 0)
+        *reinterpret_cast<float2*>(ored + (wave * G + g0 + g) * HD + dl + 2 * (lane >> 4)) = make_float2(z0, z1);
     }
   }
   __syncthreads();
@@ -835,10 +856,10 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   u16* xr = xb + xlen;                                  // residual stream        [M][D]
   float* part = reinterpret_cast<float*>(xr + M * D);   // [NW][NJMAX * M]
   float* red = part + NW * NJMAX * M;                   // [NW][M][2]
-  float* qs = red + NW * M * 2;                         // [G][HD]
+  float* qs = red + NW * M * 2;                         // [G][HD / 2] packed bf16 pairs (space for [G][HD])
   float* sc = qs + G * HD;                              // [G][sc_ld]
   float* ored = sc + G * sc_ld;                         // [NW][G][HD]
-  float* knew = ored + NW * G * HD;                     // [HD]
+  float* knew = ored + NW * G * HD;                     // [HD / 2] packed bf16 pairs (space for [HD])
   float* vnew = knew + HD;                              // [HD]
   float* s_m = vnew + HD;                               // [G]
   float* s_l = s_m + G;                                 // [G]
@@ -901,7 +922,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
                                       (p.prof && t >= p.prof_t0 && t < p.prof_t0 + PROF_SLOTS)
                                           ? p.prof + ((size_t)blockIdx.x * PROF_SLOTS + (t - p.prof_t0)) * PROF_POINTS
                                           : nullptr,
-                                      kv, qs, sc, sc_ld, ored, knew, vnew, s_m, s_l);
+                                      kv, reinterpret_cast<u32*>(qs), sc, sc_ld, ored, reinterpret_cast<u32*>(knew), vnew, s_m, s_l);
           first = false;
         }
     } else {
