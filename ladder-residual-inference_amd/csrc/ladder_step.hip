@@ -278,6 +278,8 @@ __device__ __forceinline__ void reduce8(float* v, float& z0, float& z1) {
 // Its rows are reduced in rounds of NJMAX; inside a round wave (rg, kg) owns rows j = rg (mod nrg)
 // and K-slices kk = kg (mod nkg), RB rows x one 512-element slice per unit.
 // ------------------------------------------------------------------------------------------------
+#define LR_UNI(x) __builtin_amdgcn_readfirstlane(x)
+
 struct Job {
   const u16* W;
   int K, row_base, n_items, pair_off, rpi;  // rpi: rows per item (1, or 2 for up/gate pairs)
@@ -325,96 +327,191 @@ __device__ __forceinline__ Job next_slot_job(const StepParams& p, int t, int qdi
 }
 
 struct Unit {
-  uint4 r[RB];
+  u32x4_t r[RB];
 };
 
-// Issue the loads of unit (j0, jb, kk) of `job`.  Rows beyond the round and columns beyond K are
-// clamped to valid addresses: their products are discarded / multiplied by a zero x.
-__device__ __forceinline__ void load_unit(const Job& job, int j0, int jb, int kk, int lane, Unit& u) {
+// Issue the loads of unit (j0, jb, kk) of `job`: one buffer load per row, the row's offset in a
+// scalar register, the lane's column offset shared by all rows.  Rows beyond the round and columns
+// beyond K are clamped to valid addresses: their products are discarded / multiplied by a zero x.
+// With real == false the same number of loads is issued out of the buffer's range (they return
+// zero without touching memory): the number of loads in flight then never depends on a branch.
+// That, and there being ONE load sequence in the loop (prod_issue selects the job by value), is
+// what lets the compiler's wait-count insertion wait for exactly the older unit (vmcnt(RB))
+// instead of for everything in flight.
+__device__ __forceinline__ void load_unit(const Job& job, int j0, int jb, int kk, int lane, Unit& u, bool real) {
   const int njb = job.nj - j0 < NJMAX ? job.nj - j0 : NJMAX;
   int k = kk * 512 + lane * 8;
   k = k < job.K ? k : 0;
+  const int voff = real ? k * 2 : (int)0x80000000;
+  __amdgpu_buffer_rsrc_t br = __builtin_amdgcn_make_buffer_rsrc(const_cast<u16*>(job.W), 0, job.W ? 0x7fffffff : 0, 0x00020000);
 #pragma unroll
   for (int i = 0; i < RB; ++i) {
     int j = jb + i * job.nrg;
     j = j < njb ? j : njb - 1;
     const int jj = j0 + j;
     const int row = job.row_base + job.w + job.nwg * (jj / job.rpi) + (jj % job.rpi) * job.pair_off;
-    u.r[i] = ld16(job.W + (int64_t)row * job.K + k);
+    const unsigned soff = real ? (unsigned)row * (unsigned)job.K * 2u : 0u;
+    u.r[i] = __builtin_amdgcn_raw_buffer_load_b128(br, voff, (int)LR_UNI(soff), 0);
+  }
+}
+// ---- a wave's position in the unit sequence of a job.  The sequence is: for every round, the
+//      wave's units (k-steps fastest, then row batches), padded to an even count, so that the two
+//      register sets of the pipeline alternate in a fixed way.  All of it is wave-uniform.
+struct Pos {
+  int j0, u, ur, up, jb, kk;  // round, index in the round, real / padded units of the round, coordinates
+  bool done;
+};
+__device__ __forceinline__ void pos_round(const Job& j, Pos& p) {
+  // (written without branches: every field is assigned exactly once on every path, which keeps
+  // the structure in registers)
+  const int njb = j.nj - p.j0 < NJMAX ? j.nj - p.j0 : NJMAX;
+  const bool ok = j.active && p.j0 < j.nj && j.rg < njb;
+  const int nb = (njb - j.rg + j.nrg * RB - 1) / (j.nrg * RB);
+  const int nk = (j.ksteps - j.kg + j.nkg - 1) / j.nkg;
+  const int ur = ok ? nb * nk : 0;
+  p.done = !ok;
+  p.ur = ur;
+  p.up = (ur + 1) & ~1;
+  p.u = 0;
+  p.jb = j.rg;
+  p.kk = j.kg;
+}
+__device__ __forceinline__ void pos_first(const Job& j, Pos& p) {
+  p.j0 = 0;
+  p.u = 0;
+  p.done = false;
+  pos_round(j, p);
+}
+__device__ __forceinline__ bool pos_real(const Pos& p) { return !p.done && p.u < p.ur; }
+__device__ __forceinline__ void pos_next(const Job& j, Pos& p) {
+  if (p.done) return;
+  const int u = p.u + 1;
+  if (u < p.up) {
+    int kk = p.kk, jb = p.jb;
+    if (u < p.ur) {
+      kk += j.nkg;
+      if (kk >= j.ksteps) {
+        kk = j.kg;
+        jb += j.nrg * RB;
+      }
+    }
+    p.u = u;
+    p.kk = kk;
+    p.jb = jb;
+  } else {
+    p.j0 += NJMAX;
+    pos_round(j, p);
   }
 }
 
-__device__ __forceinline__ void first_unit(const Job& job, int lane, Unit& u) {
-  if (job.active) {
-    load_unit(job, 0, job.rg, job.kg, lane, u);
-  } else {  // a defined value everywhere: ends the live range of whatever `u` held before
-#pragma unroll
-    for (int i = 0; i < RB; ++i) u.r[i] = make_uint4(0, 0, 0, 0);
+// The weight pipeline of a wave: two register sets.  While one is multiplied the other is in
+// flight, and the set just multiplied is refilled at once with the unit two positions ahead --
+// also across the end of a job, into the next one.  On entry to run_job, `a` and `b` hold the
+// wave's first two positions of that job (issued by the previous job, or by prime()).
+struct Pipe {
+  Unit a, b;
+};
+struct Prod {  // where the prefetch is: two positions ahead of the multiplier
+  Pos p;
+  bool in_next;
+};
+__device__ __forceinline__ void prod_issue(const Job& job, const Job& next, Prod& pr, int lane, Unit& u) {
+  const Job j = pr.in_next ? next : job;  // by value: scalar selects, one load sequence
+  load_unit(j, pr.p.j0, pr.p.jb, pr.p.kk, lane, u, pos_real(pr.p));
+  pos_next(j, pr.p);
+  if (pr.p.done && !pr.in_next) {
+    pr.in_next = true;
+    pos_first(next, pr.p);
   }
+}
+__device__ __forceinline__ void prime(const Job& job, int lane, Pipe& pipe) {
+  Pos p;
+  pos_first(job, p);
+  load_unit(job, p.j0, p.jb, p.kk, lane, pipe.a, pos_real(p));
+  pos_next(job, p);
+  load_unit(job, p.j0, p.jb, p.kk, lane, pipe.b, pos_real(p));
 }
 
 enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_LOGITS = 2 };
 
-// Run one job.  On entry `cur` holds this wave's first unit of the job (if it has one); on exit it
-// holds the first unit of `next` (if the wave has one there) -- issued before this job's last
-// reduction and epilogue.
+// multiply one unit into the accumulators of its row batch; at the batch's last k-step fold the
+// lanes and leave the partial sums in LDS
+template <int M>
+__device__ __forceinline__ void consume_unit(const Job& job, const Pos& c, const Unit& u, const u16* x, float* part,
+                                             float (&acc)[M][RB], int lane) {
+  const int njb = job.nj - c.j0 < NJMAX ? job.nj - c.j0 : NJMAX;
+  if (c.kk == job.kg) {
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+#pragma unroll
+      for (int i = 0; i < RB; ++i) acc[m][i] = 0.0f;
+  }
+  const int k = c.kk * 512 + lane * 8;
+  const bool kv = k < job.K;
+  float xf[M][8];
+#pragma unroll
+  for (int m = 0; m < M; ++m)
+    unpack8(kv ? *reinterpret_cast<const uint4*>(x + m * job.K + k) : make_uint4(0, 0, 0, 0), xf[m]);
+#pragma unroll
+  for (int i = 0; i < RB; ++i) {
+    float wf[8];
+    wf[0] = bf_lo(u.r[i].x); wf[1] = bf_hi(u.r[i].x); wf[2] = bf_lo(u.r[i].y); wf[3] = bf_hi(u.r[i].y);
+    wf[4] = bf_lo(u.r[i].z); wf[5] = bf_hi(u.r[i].z); wf[6] = bf_lo(u.r[i].w); wf[7] = bf_hi(u.r[i].w);
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[m][i] = fmaf(wf[e], xf[m][e], acc[m][i]);
+    __builtin_amdgcn_sched_barrier(0);  // keep the unpacked row short-lived (register pressure)
+  }
+  if (c.kk + job.nkg >= job.ksteps) {
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+#pragma unroll
+      for (int h = 0; h < RB / 8; ++h) {
+        float z0, z1;
+        reduce8(&acc[m][8 * h], z0, z1);
+        if ((lane & 15) == 0) {
+          const int r = lane >> 4;
+          const int ja = c.jb + (8 * h + 2 * r) * job.nrg, jc = c.jb + (8 * h + 2 * r + 1) * job.nrg;
+          if (ja < njb) part[(job.kg * NJMAX + ja) * M + m] = z0;
+          if (jc < njb) part[(job.kg * NJMAX + jc) * M + m] = z1;
+        }
+      }
+  }
+}
+
+// Run one job; see Pipe for what `pipe` holds on entry and on exit (`next` must be the job the
+// following run_job call is made with).
 template <int M, int EPI>
 __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, const Job& job, const Job& next,
-                                        Unit& cur, const u16* x, float* part, unsigned out_wo, int ldo, unsigned tag,
+                                        Pipe& pipe, const u16* x, float* part, unsigned out_wo, int ldo, unsigned tag,
                                         float* cand_v, int* cand_i, float* best_v, int* best_i) {
   const int tid = opaque_tid(), lane = tid & 63;
   const int RPI = job.rpi;
-  if (!job.active) first_unit(next, lane, cur);
+  if (!job.active) prime(next, lane, pipe);
+  Pos c;
+  Prod pr;
+  pos_first(job, c);
+  pr.p = c;
+  pr.in_next = false;
+  pos_next(job, pr.p);
+  pos_next(job, pr.p);
+  if (pr.p.done) {
+    pr.in_next = true;
+    pos_first(next, pr.p);
+  }
+  float acc[M][RB];
   for (int j0 = 0; j0 < job.nj; j0 += NJMAX) {
     const int njb = job.nj - j0 < NJMAX ? job.nj - j0 : NJMAX;
     if (job.active && job.rg < njb) {
-      for (int jb = job.rg; jb < njb; jb += job.nrg * RB) {
-        float acc[M][RB];
-#pragma unroll
-        for (int m = 0; m < M; ++m)
-#pragma unroll
-          for (int i = 0; i < RB; ++i) acc[m][i] = 0.0f;
-        for (int kk = job.kg; kk < job.ksteps; kk += job.nkg) {
-          // ---- put the following unit in flight
-          Unit nxt;
-          if (kk + job.nkg < job.ksteps) load_unit(job, j0, jb, kk + job.nkg, lane, nxt);
-          else if (jb + job.nrg * RB < njb) load_unit(job, j0, jb + job.nrg * RB, job.kg, lane, nxt);
-          else if (j0 + NJMAX < job.nj && job.rg < job.nj - j0 - NJMAX)
-            load_unit(job, j0 + NJMAX, job.rg, job.kg, lane, nxt);
-          else first_unit(next, lane, nxt);
-          // ---- multiply the current one
-          const int k = kk * 512 + lane * 8;
-          const bool kv = k < job.K;
-          float xf[M][8];
-#pragma unroll
-          for (int m = 0; m < M; ++m)
-            unpack8(kv ? *reinterpret_cast<const uint4*>(x + m * job.K + k) : make_uint4(0, 0, 0, 0), xf[m]);
-#pragma unroll
-          for (int i = 0; i < RB; ++i) {
-            float wf[8];
-            unpack8(cur.r[i], wf);
-#pragma unroll
-            for (int m = 0; m < M; ++m)
-#pragma unroll
-              for (int e = 0; e < 8; ++e) acc[m][i] = fmaf(wf[e], xf[m][e], acc[m][i]);
-            __builtin_amdgcn_sched_barrier(0);  // keep the unpacked row short-lived (register pressure)
-          }
-#pragma unroll
-          for (int i = 0; i < RB; ++i) cur.r[i] = nxt.r[i];
-        }
-#pragma unroll
-        for (int m = 0; m < M; ++m)
-#pragma unroll
-          for (int h = 0; h < RB / 8; ++h) {
-            float z0, z1;
-            reduce8(&acc[m][8 * h], z0, z1);
-            if ((lane & 15) == 0) {
-              const int r = lane >> 4;
-              const int ja = jb + (8 * h + 2 * r) * job.nrg, jc = jb + (8 * h + 2 * r + 1) * job.nrg;
-              if (ja < njb) part[(job.kg * NJMAX + ja) * M + m] = z0;
-              if (jc < njb) part[(job.kg * NJMAX + jc) * M + m] = z1;
-            }
-          }
+      const int up = c.up;
+      for (int u = 0; u < up; u += 2) {
+        if (pos_real(c)) consume_unit<M>(job, c, pipe.a, x, part, acc, lane);
+        prod_issue(job, next, pr, lane, pipe.a);
+        pos_next(job, c);
+        if (pos_real(c)) consume_unit<M>(job, c, pipe.b, x, part, acc, lane);
+        prod_issue(job, next, pr, lane, pipe.b);
+        pos_next(job, c);
       }
     }
     __syncthreads();
@@ -888,8 +985,8 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   const int k1 = k0 + chunk < nkeys ? k0 + chunk : nkeys;
 
   const int qdim = Hq * HD;
-  Unit cur;
-  first_unit(slot_job(p, 0, 0, qdim, w, nwg, wave), lane, cur);
+  Pipe pipe;
+  prime(slot_job(p, 0, 0, qdim, w, nwg, wave), lane, pipe);
 
 #define LR_STAMP(k)                                                                                  \
   if (p.prof && t >= p.prof_t0 && t < p.prof_t0 + PROF_SLOTS && tid == 0)                            \
@@ -909,7 +1006,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
     if (tid == 0) coh.st(p.odone + (unsigned)w, 0.0f, tag);
     LR_STAMP(1)
     if (has_a && att_wg) {
-      run_job<M, EPI_STORE>(p, coh, LR_JOB(0), LR_JOB(2), cur, xa, part, p.oqkv, p.nqkv, tag, nullptr, nullptr,
+      run_job<M, EPI_STORE>(p, coh, LR_JOB(0), LR_JOB(2), pipe, xa, part, p.oqkv, p.nqkv, tag, nullptr, nullptr,
                             nullptr, nullptr);
       LR_STAMP(2)
       // ---------------- attention workgroup (it owns no rows of w1)
@@ -926,20 +1023,23 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
           first = false;
         }
     } else {
-      run_job<M, EPI_STORE>(p, coh, LR_JOB(0), LR_JOB(1), cur, xa, part, p.oqkv, p.nqkv, tag, nullptr, nullptr,
+      run_job<M, EPI_STORE>(p, coh, LR_JOB(0), LR_JOB(1), pipe, xa, part, p.oqkv, p.nqkv, tag, nullptr, nullptr,
                             nullptr, nullptr);
       LR_STAMP(2)
       // ---------------- everyone else: the up/gate projection of the previous layer + SwiGLU
-      run_job<M, EPI_SWIGLU>(p, coh, LR_JOB(1), has_a ? LR_JOB(2) : LR_JOB(3), cur, xb, part, act_wo, I, tag, nullptr,
-                             nullptr, nullptr, nullptr);
+      const Job after_w1 = LR_JOB(has_a ? 2 : 3);  // named values, not conditional temporaries: they stay in registers
+      run_job<M, EPI_SWIGLU>(p, coh, LR_JOB(1), after_w1, pipe, xb, part, act_wo, I, tag, nullptr, nullptr, nullptr,
+                             nullptr);
     }
     LR_STAMP(3)
     // ---------------- merge attention partials, output projection
     if (has_a) {
       attention_merge<M, HD>(p, coh, Hq, tag, xa, wbuf);
       LR_STAMP(4)
-      run_job<M, EPI_STORE>(p, coh, LR_JOB(2), has_b ? LR_JOB(3) : next_slot_job(p, t, qdim, w, nwg, wave), cur, xa,
-                            part, p.oa, D, tag, nullptr, nullptr, nullptr, nullptr);
+      Job after_wo = next_slot_job(p, t, qdim, w, nwg, wave);
+      if (has_b) after_wo = LR_JOB(3);
+      run_job<M, EPI_STORE>(p, coh, LR_JOB(2), after_wo, pipe, xa, part, p.oa, D, tag, nullptr, nullptr, nullptr,
+                            nullptr);
     } else if (has_b) {
       // no attention in this slot, hence nobody has checked the "done" words yet: do it here,
       // before the down projection overwrites m
@@ -950,7 +1050,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
     if (has_b) {
       load_x<M>(coh, act_wo, tag, I, xb);
       LR_STAMP(6)
-      run_job<M, EPI_STORE>(p, coh, LR_JOB(3), next_slot_job(p, t, qdim, w, nwg, wave), cur, xb, part, p.om, D, tag,
+      run_job<M, EPI_STORE>(p, coh, LR_JOB(3), next_slot_job(p, t, qdim, w, nwg, wave), pipe, xb, part, p.om, D, tag,
                             nullptr, nullptr, nullptr, nullptr);
     }
     LR_STAMP(7)
@@ -967,7 +1067,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
               p.final_norm, xb, xa, red);
   float best_v = -INFINITY;
   int best_i = 0x7fffffff;
-  run_job<M, EPI_LOGITS>(p, coh, slot_job(p, 4, L + 1, qdim, w, nwg, wave), slot_job(p, -1, 0, qdim, w, nwg, wave), cur,
+  run_job<M, EPI_LOGITS>(p, coh, slot_job(p, 4, L + 1, qdim, w, nwg, wave), slot_job(p, -1, 0, qdim, w, nwg, wave), pipe,
                          xa, part, 0u, 0, tag,
                          cand_v, cand_i, &best_v, &best_i);
   if (tid < M) {  // candidate: value (bf16-exact), a filler word, index as two 16-bit halves
