@@ -230,6 +230,12 @@ __device__ __forceinline__ void f32x2_from(const u32x4_t& a, float& v0, float& v
   v1 = __uint_as_float((a.z & 0xffff0000u) | (a.w >> 16));
 }
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+// c + a.lo * b.lo + a.hi * b.hi on packed bf16 pairs, fp32 accumulation
+__device__ __forceinline__ float dot2(u32 a, u32 b, float c) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
+}
+
 // ---- per-lane accumulators -> wave totals.  reduce8: afterwards lane 16*r holds sum(v[2r]) in z0
 //      and sum(v[2r+1]) in z1.  (permlane swaps fold halves / odd-even rows, DPP folds a row.)
 __device__ __forceinline__ void swap32(float& a, float& b) {
@@ -280,50 +286,92 @@ __device__ __forceinline__ void reduce8(float* v, float& z0, float& z1) {
 // ------------------------------------------------------------------------------------------------
 #define LR_UNI(x) __builtin_amdgcn_readfirstlane(x)
 
-struct Job {
-  const u16* W;
-  int K, row_base, n_items, pair_off, rpi;  // rpi: rows per item (1, or 2 for up/gate pairs)
-  int w, nwg;                               // this workgroup's rank among the participants
-  int nj, ksteps, nkg, nrg, rg, kg;         // derived for this workgroup / wave
-  bool active;
-};
+// Everything about a job that does not change from layer to layer (all but the matrix pointer) is
+// worked out once per launch, per job kind and wave, and kept in LDS: the per-layer code then has
+// no divisions and little scalar state (a wave issues at most one instruction every four cycles,
+// so bookkeeping instructions are what small jobs are made of).
+enum { JK_QKV = 0, JK_W1_SPLIT, JK_WO, JK_W2, JK_HEAD, JK_W1_ALL, JK_NONE, JK_COUNT };
 
-__device__ __forceinline__ Job make_job(const u16* W, int K, int row_base, int n_items, int pair_off, int rpi,
-                                        int w, int nwg, int wave) {
+struct Job {  // wave-uniform
+  int K2;                  // bytes per row
+  int pair_off, rsh;       // item -> rows: row = w + nwg * (jj >> rsh) + (jj & rsh) * pair_off   (rsh 0 or 1)
+  int w, nwg;              // this workgroup's rank among the participants
+  int nj;                  // rows this workgroup owns
+  int ksteps, nkg, nrg;    // 512-element K slices; waves along K; waves along rows
+  int rg, kg;              // this wave's place
+  int nk;                  // k-steps per row batch for this wave
+  int bsh;                 // log2(nrg * RB): row stride between a wave's batches
+  int active;              // this wave has work in the job
+  int K;
+  int _pad;
+  const u16* W;            // not in LDS: set per layer
+};
+static_assert(sizeof(Job) == 16 * 4 + 8, "16 table words + the pointer");
+
+__device__ __forceinline__ void build_job(int* rec, int K, int n_items, int pair_off, int rsh, int w, int nwg,
+                                          int wave) {
   Job j;
-  j.W = W; j.K = K; j.row_base = row_base; j.n_items = n_items; j.pair_off = pair_off; j.rpi = rpi;
-  j.w = w; j.nwg = nwg;
-  const int nit = (W != nullptr && w >= 0 && n_items > w) ? (n_items - w + nwg - 1) / nwg : 0;
-  j.nj = nit * rpi;
+  j.K = K; j.K2 = K * 2; j.pair_off = pair_off; j.rsh = rsh; j.w = w; j.nwg = nwg;
+  const int nit = (w >= 0 && n_items > w) ? (n_items - w + nwg - 1) / nwg : 0;
+  j.nj = nit << rsh;
   j.ksteps = (K + 511) >> 9;
   j.nkg = j.ksteps < NW ? j.ksteps : NW;
   j.nrg = NW / j.nkg;
   j.rg = wave / j.nkg;
   j.kg = wave - j.rg * j.nkg;
-  j.active = wave < j.nrg * j.nkg && j.rg < (j.nj < NJMAX ? j.nj : NJMAX);
+  j.active = (wave < j.nrg * j.nkg && j.rg < (j.nj < NJMAX ? j.nj : NJMAX)) ? 1 : 0;
+  j.nk = j.kg < j.ksteps ? (j.ksteps - j.kg + j.nkg - 1) / j.nkg : 0;
+  j.bsh = 31 - __builtin_clz(j.nrg * RB);
+  j._pad = 0;
+  const int* src = reinterpret_cast<const int*>(&j);
+  for (int i = 0; i < 16; ++i) rec[i] = src[i];
+}
+
+// table: [JK_COUNT][NW][16] ints in LDS, filled once per launch
+__device__ __forceinline__ void build_job_table(const StepParams& p, int* table, int qdim, int w, int nwg) {
+  const int i = threadIdx.x;
+  if (i < JK_COUNT * NW) {
+    const int kind = i / NW, wave = i - kind * NW;
+    int* rec = table + i * 16;
+    if (kind == JK_QKV) build_job(rec, p.D, p.nqkv, 0, 0, w, nwg, wave);
+    else if (kind == JK_W1_SPLIT) build_job(rec, p.D, p.I, p.I, 1, w - p.NA, nwg - p.NA, wave);
+    else if (kind == JK_WO) build_job(rec, qdim, p.D, 0, 0, w, nwg, wave);
+    else if (kind == JK_W2) build_job(rec, p.I, p.D, 0, 0, w, nwg, wave);
+    else if (kind == JK_HEAD) build_job(rec, p.D, p.V, 0, 0, w, nwg, wave);
+    else if (kind == JK_W1_ALL) build_job(rec, p.D, p.I, p.I, 1, w, nwg, wave);
+    else build_job(rec, 512, 0, 0, 0, 0, 1, wave);
+  }
+}
+
+__device__ __forceinline__ Job load_job(const int* table, int kind, int wave, const u16* W) {
+  const int4* r = reinterpret_cast<const int4*>(table + (kind * NW + wave) * 16);
+  const int4 a = r[0], b = r[1], c = r[2], d = r[3];
+  Job j;
+  j.K2 = LR_UNI(a.x); j.pair_off = LR_UNI(a.y); j.rsh = LR_UNI(a.z); j.w = LR_UNI(a.w);
+  j.nwg = LR_UNI(b.x); j.nj = LR_UNI(b.y); j.ksteps = LR_UNI(b.z); j.nkg = LR_UNI(b.w);
+  j.nrg = LR_UNI(c.x); j.rg = LR_UNI(c.y); j.kg = LR_UNI(c.z); j.nk = LR_UNI(c.w);
+  j.bsh = LR_UNI(d.x); j.active = LR_UNI(d.y); j.K = LR_UNI(d.z); j._pad = 0;
+  j.W = W;
   return j;
 }
 
-// The jobs of slot t, built where they are needed (few are alive at a time: they live in scalar
-// registers).  kind: 0 wqkv(t), 1 w1(t-1), 2 wo(t), 3 w2(t-1), 4 lm_head; a slot without that
-// module gets a job that owns no rows.  w1 is dealt to the workgroups that do not run attention
-// in the slot.
-__device__ __forceinline__ Job slot_job(const StepParams& p, int kind, int t, int qdim, int w, int nwg, int wave) {
+// The jobs of slot t.  kind: 0 wqkv(t), 1 w1(t-1), 2 wo(t), 3 w2(t-1), 4 lm_head; a slot without
+// that module gets a job that owns no rows.  w1 is dealt to the workgroups that do not run
+// attention in the slot.
+__device__ __forceinline__ Job slot_job(const StepParams& p, const int* table, int kind, int t, int wave) {
   const bool a = t < p.L, b = t >= 1 && t <= p.L;
-  if (kind == 0 && a) return make_job(p.layers[t].wqkv, p.D, 0, p.nqkv, 0, 1, w, nwg, wave);
-  if (kind == 1 && b)
-    return a ? make_job(p.layers[t - 1].w1, p.D, 0, p.I, p.I, 2, w - p.NA, nwg - p.NA, wave)
-             : make_job(p.layers[t - 1].w1, p.D, 0, p.I, p.I, 2, w, nwg, wave);
-  if (kind == 2 && a) return make_job(p.layers[t].wo, qdim, 0, p.D, 0, 1, w, nwg, wave);
-  if (kind == 3 && b) return make_job(p.layers[t - 1].w2, p.I, 0, p.D, 0, 1, w, nwg, wave);
-  if (kind == 4) return make_job(p.out_w, p.D, 0, p.V, 0, 1, w, nwg, wave);
-  return make_job(nullptr, 512, 0, 0, 0, 1, 0, 1, wave);
+  int jk = JK_NONE;
+  const u16* W = nullptr;
+  if (kind == 0 && a) { jk = JK_QKV; W = p.layers[t].wqkv; }
+  if (kind == 1 && b) { jk = a ? JK_W1_SPLIT : JK_W1_ALL; W = p.layers[t - 1].w1; }
+  if (kind == 2 && a) { jk = JK_WO; W = p.layers[t].wo; }
+  if (kind == 3 && b) { jk = JK_W2; W = p.layers[t - 1].w2; }
+  if (kind == 4) { jk = JK_HEAD; W = p.out_w; }
+  return load_job(table, jk, wave, W);
 }
 // first job of slot t + 1
-__device__ __forceinline__ Job next_slot_job(const StepParams& p, int t, int qdim, int w, int nwg, int wave) {
-  if (t + 1 < p.L) return slot_job(p, 0, t + 1, qdim, w, nwg, wave);
-  if (t + 1 == p.L) return slot_job(p, 1, t + 1, qdim, w, nwg, wave);
-  return slot_job(p, 4, t + 1, qdim, w, nwg, wave);
+__device__ __forceinline__ Job next_slot_job(const StepParams& p, const int* table, int t, int wave) {
+  return slot_job(p, table, t + 1 < p.L ? 0 : (t + 1 == p.L ? 1 : 4), t + 1, wave);
 }
 
 struct Unit {
@@ -343,14 +391,15 @@ __device__ __forceinline__ void load_unit(const Job& job, int j0, int jb, int kk
   int k = kk * 512 + lane * 8;
   k = k < job.K ? k : 0;
   const int voff = real ? k * 2 : (int)0x80000000;
+  const int rmask = (1 << job.rsh) - 1;
   __amdgpu_buffer_rsrc_t br = __builtin_amdgcn_make_buffer_rsrc(const_cast<u16*>(job.W), 0, job.W ? 0x7fffffff : 0, 0x00020000);
 #pragma unroll
   for (int i = 0; i < RB; ++i) {
     int j = jb + i * job.nrg;
     j = j < njb ? j : njb - 1;
     const int jj = j0 + j;
-    const int row = job.row_base + job.w + job.nwg * (jj / job.rpi) + (jj % job.rpi) * job.pair_off;
-    const unsigned soff = real ? (unsigned)row * (unsigned)job.K * 2u : 0u;
+    const int row = job.w + job.nwg * (jj >> job.rsh) + (jj & rmask) * job.pair_off;
+    const unsigned soff = real ? (unsigned)row * (unsigned)job.K2 : 0u;
     u.r[i] = __builtin_amdgcn_raw_buffer_load_b128(br, voff, (int)LR_UNI(soff), 0);
   }
 }
@@ -366,9 +415,8 @@ __device__ __forceinline__ void pos_round(const Job& j, Pos& p) {
   // the structure in registers)
   const int njb = j.nj - p.j0 < NJMAX ? j.nj - p.j0 : NJMAX;
   const bool ok = j.active && p.j0 < j.nj && j.rg < njb;
-  const int nb = (njb - j.rg + j.nrg * RB - 1) / (j.nrg * RB);
-  const int nk = (j.ksteps - j.kg + j.nkg - 1) / j.nkg;
-  const int ur = ok ? nb * nk : 0;
+  const int nb = (njb - j.rg + (1 << j.bsh) - 1) >> j.bsh;
+  const int ur = ok ? nb * j.nk : 0;
   p.done = !ok;
   p.ur = ur;
   p.up = (ur + 1) & ~1;
@@ -392,7 +440,7 @@ __device__ __forceinline__ void pos_next(const Job& j, Pos& p) {
       kk += j.nkg;
       if (kk >= j.ksteps) {
         kk = j.kg;
-        jb += j.nrg * RB;
+        jb += 1 << j.bsh;
       }
     }
     p.u = u;
@@ -413,14 +461,15 @@ struct Pipe {
 };
 struct Prod {  // where the prefetch is: two positions ahead of the multiplier
   Pos p;
+  Job job;  // the job it is walking (this one, later the next)
   bool in_next;
 };
-__device__ __forceinline__ void prod_issue(const Job& job, const Job& next, Prod& pr, int lane, Unit& u) {
-  const Job j = pr.in_next ? next : job;  // by value: scalar selects, one load sequence
-  load_unit(j, pr.p.j0, pr.p.jb, pr.p.kk, lane, u, pos_real(pr.p));
-  pos_next(j, pr.p);
+__device__ __forceinline__ void prod_issue(const Job& next, Prod& pr, int lane, Unit& u) {
+  load_unit(pr.job, pr.p.j0, pr.p.jb, pr.p.kk, lane, u, pos_real(pr.p));  // the ONE load sequence of the loop
+  pos_next(pr.job, pr.p);
   if (pr.p.done && !pr.in_next) {
     pr.in_next = true;
+    pr.job = next;
     pos_first(next, pr.p);
   }
 }
@@ -448,20 +497,22 @@ __device__ __forceinline__ void consume_unit(const Job& job, const Pos& c, const
   }
   const int k = c.kk * 512 + lane * 8;
   const bool kv = k < job.K;
-  float xf[M][8];
+  // weights and inputs stay packed bf16 pairs: one v_dot2_f32_bf16 per pair of products (fp32 sums)
+  uint4 xp[M];
 #pragma unroll
   for (int m = 0; m < M; ++m)
-    unpack8(kv ? *reinterpret_cast<const uint4*>(x + m * job.K + k) : make_uint4(0, 0, 0, 0), xf[m]);
+    xp[m] = kv ? *reinterpret_cast<const uint4*>(x + m * job.K + k) : make_uint4(0, 0, 0, 0);
 #pragma unroll
   for (int i = 0; i < RB; ++i) {
-    float wf[8];
-    wf[0] = bf_lo(u.r[i].x); wf[1] = bf_hi(u.r[i].x); wf[2] = bf_lo(u.r[i].y); wf[3] = bf_hi(u.r[i].y);
-    wf[4] = bf_lo(u.r[i].z); wf[5] = bf_hi(u.r[i].z); wf[6] = bf_lo(u.r[i].w); wf[7] = bf_hi(u.r[i].w);
 #pragma unroll
-    for (int m = 0; m < M; ++m)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[m][i] = fmaf(wf[e], xf[m][e], acc[m][i]);
-    __builtin_amdgcn_sched_barrier(0);  // keep the unpacked row short-lived (register pressure)
+    for (int m = 0; m < M; ++m) {
+      float a = acc[m][i];
+      a = dot2(u.r[i].x, xp[m].x, a);
+      a = dot2(u.r[i].y, xp[m].y, a);
+      a = dot2(u.r[i].z, xp[m].z, a);
+      a = dot2(u.r[i].w, xp[m].w, a);
+      acc[m][i] = a;
+    }
   }
   if (c.kk + job.nkg >= job.ksteps) {
 #pragma unroll
@@ -487,17 +538,19 @@ __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, con
                                         Pipe& pipe, const u16* x, float* part, unsigned out_wo, int ldo, unsigned tag,
                                         float* cand_v, int* cand_i, float* best_v, int* best_i) {
   const int tid = opaque_tid(), lane = tid & 63;
-  const int RPI = job.rpi;
+  const int RPI = 1 << job.rsh;
   if (!job.active) prime(next, lane, pipe);
   Pos c;
   Prod pr;
   pos_first(job, c);
   pr.p = c;
+  pr.job = job;
   pr.in_next = false;
   pos_next(job, pr.p);
   pos_next(job, pr.p);
   if (pr.p.done) {
     pr.in_next = true;
+    pr.job = next;
     pos_first(next, pr.p);
   }
   float acc[M][RB];
@@ -507,16 +560,16 @@ __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, con
       const int up = c.up;
       for (int u = 0; u < up; u += 2) {
         if (pos_real(c)) consume_unit<M>(job, c, pipe.a, x, part, acc, lane);
-        prod_issue(job, next, pr, lane, pipe.a);
+        prod_issue(next, pr, lane, pipe.a);
         pos_next(job, c);
         if (pos_real(c)) consume_unit<M>(job, c, pipe.b, x, part, acc, lane);
-        prod_issue(job, next, pr, lane, pipe.b);
+        prod_issue(next, pr, lane, pipe.b);
         pos_next(job, c);
       }
     }
     __syncthreads();
     // ---- cross-wave sum in fixed order + epilogue
-    const int nout = (njb / RPI) * M;
+    const int nout = (njb >> job.rsh) * M;
     if (tid < nout) {
       const int jl = tid / M, m = tid - jl * M;
       float s0, s1 = 0.0f;
@@ -530,7 +583,7 @@ __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, con
         for (int g = 0; g < job.nkg; ++g) t += part[(g * NJMAX + jl * RPI + 1) * M + m];
         s1 = round_bf(t);
       }
-      const int it = job.w + job.nwg * ((j0 / RPI) + jl);
+      const int it = job.w + job.nwg * ((j0 >> job.rsh) + jl);
       if (m < p.B) {
         if (EPI == EPI_STORE) coh.st(out_wo + (unsigned)(m * ldo + it), s0, tag);
         if (EPI == EPI_SWIGLU) coh.st(out_wo + (unsigned)(m * ldo + it), swiglu_bf(s0, s1), tag);
@@ -684,12 +737,6 @@ __device__ __forceinline__ void load_x(const Coh& coh, unsigned src_wo, unsigned
 // softmax and P.V stay in fp32; each workgroup publishes an un-normalised partial result with its
 // own (max, sum) as tagged fp32 word pairs.
 // ------------------------------------------------------------------------------------------------
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-// c + a.lo * b.lo + a.hi * b.hi on packed bf16 pairs, fp32 accumulation
-__device__ __forceinline__ float dot2(u32 a, u32 b, float c) {
-  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
-}
-
 __device__ __forceinline__ void rope_pair(float x0, float x1, float c, float s, float& o0, float& o1) {
 #pragma clang fp contract(off)
   const float a = x0 * c, b = x1 * s, d = x1 * c, e = x0 * s;
@@ -964,6 +1011,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   float* cand_v = wbuf + M * Hq * NA_MAX;               // [NJMAX * M]
   int* cand_i = reinterpret_cast<int*>(cand_v + NJMAX * M);
   int* s_flag = cand_i + NJMAX * M;                     // [8]
+  int* jtab = s_flag + 8;                               // [JK_COUNT][NW][16] job table
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -973,6 +1021,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   coh.r = __builtin_amdgcn_make_buffer_rsrc(p.ws, 0, (int)p.ws_bytes, 0x00020000);
   coh.fail = &ctrl->fail;
   if (tid == 0) s_flag[1] = (int)cldu(&ctrl->epoch_base);
+  build_job_table(p, jtab, Hq * HD, w, nwg);
   __syncthreads();
   const unsigned epoch_base = (unsigned)s_flag[1];
   int pos = p.pos[0];
@@ -986,12 +1035,12 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
 
   const int qdim = Hq * HD;
   Pipe pipe;
-  prime(slot_job(p, 0, 0, qdim, w, nwg, wave), lane, pipe);
+  prime(slot_job(p, jtab, 0, 0, wave), lane, pipe);
 
 #define LR_STAMP(k)                                                                                  \
   if (p.prof && t >= p.prof_t0 && t < p.prof_t0 + PROF_SLOTS && tid == 0)                            \
     p.prof[((size_t)blockIdx.x * PROF_SLOTS + (t - p.prof_t0)) * PROF_POINTS + (k)] = wall_clock64();
-#define LR_JOB(kind) slot_job(p, kind, t, qdim, w, nwg, wave)
+#define LR_JOB(kind) slot_job(p, jtab, kind, t, wave)
   for (int t = 0; t <= L; ++t) {
     const bool has_a = t < L, has_b = t >= 1;
     const LayerPtrs* la = p.layers + (has_a ? t : L - 1);
@@ -1036,7 +1085,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
     if (has_a) {
       attention_merge<M, HD>(p, coh, Hq, tag, xa, wbuf);
       LR_STAMP(4)
-      Job after_wo = next_slot_job(p, t, qdim, w, nwg, wave);
+      Job after_wo = next_slot_job(p, jtab, t, wave);
       if (has_b) after_wo = LR_JOB(3);
       run_job<M, EPI_STORE>(p, coh, LR_JOB(2), after_wo, pipe, xa, part, p.oa, D, tag, nullptr, nullptr, nullptr,
                             nullptr);
@@ -1050,7 +1099,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
     if (has_b) {
       load_x<M>(coh, act_wo, tag, I, xb);
       LR_STAMP(6)
-      run_job<M, EPI_STORE>(p, coh, LR_JOB(3), next_slot_job(p, t, qdim, w, nwg, wave), pipe, xb, part, p.om, D, tag,
+      run_job<M, EPI_STORE>(p, coh, LR_JOB(3), next_slot_job(p, jtab, t, wave), pipe, xb, part, p.om, D, tag,
                             nullptr, nullptr, nullptr, nullptr);
     }
     LR_STAMP(7)
@@ -1067,7 +1116,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
               p.final_norm, xb, xa, red);
   float best_v = -INFINITY;
   int best_i = 0x7fffffff;
-  run_job<M, EPI_LOGITS>(p, coh, slot_job(p, 4, L + 1, qdim, w, nwg, wave), slot_job(p, -1, 0, qdim, w, nwg, wave), pipe,
+  run_job<M, EPI_LOGITS>(p, coh, slot_job(p, jtab, 4, L + 1, wave), slot_job(p, jtab, -1, 0, wave), pipe,
                          xa, part, 0u, 0, tag,
                          cand_v, cand_i, &best_v, &best_i);
   if (tid < M) {  // candidate: value (bf16-exact), a filler word, index as two 16-bit halves
@@ -1189,7 +1238,7 @@ template <int M, int HD, int G>
 static size_t lds_bytes(int D, int I, int Hq) {
   const int xlen = M * (D > I ? D : I);
   const size_t fl = (size_t)NW * NJMAX * M + NW * M * 2 + G * HD + (size_t)G * att_capacity(HD) + NW * G * HD +
-                    2 * HD + 2 * G + (size_t)M * Hq * NA_MAX + 2 * NJMAX * M + 8;
+                    2 * HD + 2 * G + (size_t)M * Hq * NA_MAX + 2 * NJMAX * M + 8 + JK_COUNT * NW * 16;
   return ((size_t)xlen * 2 + (size_t)M * D) * sizeof(u16) + fl * sizeof(float) + 16;
 }
 
