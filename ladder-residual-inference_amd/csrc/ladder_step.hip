@@ -744,24 +744,30 @@ __device__ __forceinline__ void rope_pair(float x0, float x1, float c, float s, 
   o1 = round_bf(d + e);
 }
 
+constexpr int ATT_KT = 2;  // 32-key tiles of K an attention wave keeps in registers (MFMA operand layout)
+template <int HD>
 struct KV {
-  uint4 k[ATT_NI], v[ATT_NI];
+  uint4 k[ATT_KT][HD / 16];  // tile t, k-step s: key = lane % 32 of the tile, elements s * 16 + (lane / 32) * 8 .. + 8
+  uint4 v[ATT_NI];           // key group layout (see attention_load)
 };
 
 template <int HD>
 __device__ __forceinline__ void attention_load(const StepParams& p, const LayerPtrs& lp, int b, int kvh, int k0,
-                                               int k1, int pos, KV& kv) {
+                                               int k1, int pos, KV<HD>& kv) {
   constexpr int LPK = HD / 8, KPW = 64 / LPK;
   const int tid_ = opaque_tid();
   const int wave = tid_ >> 6, lane = tid_ & 63;
   const int kl = lane / LPK, dl = (lane % LPK) * 8;
   const u16* kbase = lp.k_cache + ((int64_t)b * p.Hkv + kvh) * p.Smax * HD;
   const u16* vbase = lp.v_cache + ((int64_t)b * p.Hkv + kvh) * p.Smax * HD;
+  // K: tile (wave + NW * t) of 32 keys; a lane holds, per k-step, the 8 elements the MFMA wants from it
 #pragma unroll
-  for (int i = 0; i < ATT_NI; ++i) {
-    const int key = k0 + (i * NW + wave) * KPW + kl;
+  for (int t = 0; t < ATT_KT; ++t) {
+    const int key = k0 + (t * NW + wave) * 32 + (lane & 31);
     const bool live = key < k1 && key != pos;  // the slot of `pos` is filled from this step's qkv
-    kv.k[i] = live ? ld16(kbase + (int64_t)key * HD + dl) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int s = 0; s < HD / 16; ++s)
+      kv.k[t][s] = live ? ld16(kbase + (int64_t)key * HD + s * 16 + (lane >> 5) * 8) : make_uint4(0, 0, 0, 0);
   }
 #pragma unroll
   for (int i = 0; i < ATT_NI; ++i) {
@@ -775,7 +781,7 @@ template <int M, int HD, int G>
 __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh& coh, const LayerPtrs& lp, int b,
                                                   int kvh, int k0, int k1, int pos, unsigned tag, bool poll_done,
                                                   unsigned long long* stamp,
-                                                  KV& kv, u32* qp,
+                                                  KV<HD>& kv, u32* qp,
                                                   float* sc, int sc_ld, float* ored, u32* kp, float* vnew,
                                                   float* s_m, float* s_l) {
   constexpr int LPK = HD / 8, KPW = 64 / LPK;
@@ -847,22 +853,34 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
     __syncthreads();
     return;
   }
-  // ---- scores: K and q are bf16 pairs, so a pair of products per v_dot2_f32_bf16 (fp32 sums)
+  // ---- scores on the matrix cores: S[key][head] = sum_d K[key][d] q[head][d], one 32 x 32 tile per
+  //      32 keys (columns beyond the G heads multiply zeros), HD / 16 v_mfma_f32_32x32x16_bf16 each
 #pragma unroll
-  for (int i = 0; i < ATT_NI; ++i) {
-    if (i * NW * KPW < n) {  // uniform: later iterations hold no key of this range
-      const int key = k0 + (i * NW + wave) * KPW + kl;
-      uint4 kk = kv.k[i];
-      if (key == pos) kk = *reinterpret_cast<const uint4*>(kp + dl / 2);
+  for (int t = 0; t < ATT_KT; ++t) {
+    const int tile0 = (t * NW + wave) * 32;
+    if (tile0 < n) {  // uniform
+      const int key = k0 + tile0 + (lane & 31);
+      const int g = lane & 31;
+      f32x16_t acc;
 #pragma unroll
-      for (int g = 0; g < G; ++g) {
-        const uint4 q4 = *reinterpret_cast<const uint4*>(qp + g * (HD / 2) + dl / 2);
-        float s = dot2(kk.x, q4.x, 0.0f);
-        s = dot2(kk.y, q4.y, s);
-        s = dot2(kk.z, q4.z, s);
-        s = dot2(kk.w, q4.w, s);
-        s = LPK == 16 ? row_sum16(s) : half_row_sum8(s);
-        if (key < k1 && (lane % LPK) == 0) sc[g * sc_ld + key - k0] = s * scale;
+      for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+#pragma unroll
+      for (int s = 0; s < HD / 16; ++s) {
+        const int e0 = s * 16 + (lane >> 5) * 8;
+        uint4 ka = kv.k[t][s];
+        if (key == pos) ka = *reinterpret_cast<const uint4*>(kp + e0 / 2);
+        const uint4 qb = g < G ? *reinterpret_cast<const uint4*>(qp + g * (HD / 2) + e0 / 2) : make_uint4(0, 0, 0, 0);
+        const u32x4_t kav = {ka.x, ka.y, ka.z, ka.w}, qbv = {qb.x, qb.y, qb.z, qb.w};
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kav), __builtin_bit_cast(bf16x8_t, qbv),
+                                                      acc, 0, 0, 0);
+      }
+      // accumulator element v: key row (v / 4) * 8 + (lane / 32) * 4 + v % 4, head column lane % 32
+      if (g < G) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int kr = tile0 + (v / 4) * 8 + (lane >> 5) * 4 + (v % 4);
+          if (kr < n) sc[g * sc_ld + kr] = acc[v] * scale;
+        }
       }
     }
   }
@@ -1059,7 +1077,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
                             nullptr, nullptr);
       LR_STAMP(2)
       // ---------------- attention workgroup (it owns no rows of w1)
-      KV kv;
+      KV<HD> kv;
       bool first = true;
       for (int b = 0; b < p.B; ++b)
         for (int kvh = 0; kvh < p.Hkv; ++kvh) {
