@@ -101,6 +101,12 @@ __device__ __forceinline__ int opaque_tid() {
   return t;
 }
 
+// Workgroup barrier for data exchanged through LDS.  __syncthreads() also waits for every global
+// load of the wave (vmcnt(0)), i.e. for the weight units just requested for later -- a full memory
+// round trip at every reduction.  Waves of a workgroup only ever talk through LDS here, so waiting
+// for the LDS operations is enough.
+__device__ __forceinline__ void wg_sync() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 __device__ __forceinline__ unsigned cldu(const unsigned* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -303,12 +309,13 @@ struct Job {  // wave-uniform
   int bsh;                 // log2(nrg * RB): row stride between a wave's batches
   int active;              // this wave has work in the job
   int K;
-  int _pad;
+  int kind;                // JK_*: selects the row-offset table
   const u16* W;            // not in LDS: set per layer
+  const int* rowtab;       // not in LDS: row offsets of the first round (see build_row_table)
 };
-static_assert(sizeof(Job) == 16 * 4 + 8, "16 table words + the pointer");
+static_assert(sizeof(Job) == 16 * 4 + 16, "16 table words + two pointers");
 
-__device__ __forceinline__ void build_job(int* rec, int K, int n_items, int pair_off, int rsh, int w, int nwg,
+__device__ __forceinline__ void build_job(int* rec, int kind, int K, int n_items, int pair_off, int rsh, int w, int nwg,
                                           int wave) {
   Job j;
   j.K = K; j.K2 = K * 2; j.pair_off = pair_off; j.rsh = rsh; j.w = w; j.nwg = nwg;
@@ -322,7 +329,7 @@ __device__ __forceinline__ void build_job(int* rec, int K, int n_items, int pair
   j.active = (wave < j.nrg * j.nkg && j.rg < (j.nj < NJMAX ? j.nj : NJMAX)) ? 1 : 0;
   j.nk = j.kg < j.ksteps ? (j.ksteps - j.kg + j.nkg - 1) / j.nkg : 0;
   j.bsh = 31 - __builtin_clz(j.nrg * RB);
-  j._pad = 0;
+  j.kind = kind;
   const int* src = reinterpret_cast<const int*>(&j);
   for (int i = 0; i < 16; ++i) rec[i] = src[i];
 }
@@ -333,13 +340,34 @@ __device__ __forceinline__ void build_job_table(const StepParams& p, int* table,
   if (i < JK_COUNT * NW) {
     const int kind = i / NW, wave = i - kind * NW;
     int* rec = table + i * 16;
-    if (kind == JK_QKV) build_job(rec, p.D, p.nqkv, 0, 0, w, nwg, wave);
-    else if (kind == JK_W1_SPLIT) build_job(rec, p.D, p.I, p.I, 1, w - p.NA, nwg - p.NA, wave);
-    else if (kind == JK_WO) build_job(rec, qdim, p.D, 0, 0, w, nwg, wave);
-    else if (kind == JK_W2) build_job(rec, p.I, p.D, 0, 0, w, nwg, wave);
-    else if (kind == JK_HEAD) build_job(rec, p.D, p.V, 0, 0, w, nwg, wave);
-    else if (kind == JK_W1_ALL) build_job(rec, p.D, p.I, p.I, 1, w, nwg, wave);
-    else build_job(rec, 512, 0, 0, 0, 0, 1, wave);
+    if (kind == JK_QKV) build_job(rec, kind, p.D, p.nqkv, 0, 0, w, nwg, wave);
+    else if (kind == JK_W1_SPLIT) build_job(rec, kind, p.D, p.I, p.I, 1, w - p.NA, nwg - p.NA, wave);
+    else if (kind == JK_WO) build_job(rec, kind, qdim, p.D, 0, 0, w, nwg, wave);
+    else if (kind == JK_W2) build_job(rec, kind, p.I, p.D, 0, 0, w, nwg, wave);
+    else if (kind == JK_HEAD) build_job(rec, kind, p.D, p.V, 0, 0, w, nwg, wave);
+    else if (kind == JK_W1_ALL) build_job(rec, kind, p.D, p.I, p.I, 1, w, nwg, wave);
+    else build_job(rec, kind, 512, 0, 0, 0, 0, 1, wave);
+  }
+}
+
+// Byte offsets of the rows of a job's FIRST round, per kind, ordered so that the RB rows of one
+// unit are consecutive: entry ((rg * (64 >> bsh)) + batch) * RB + i is row j = rg + (batch << bsh) +
+// i * nrg of the round, clamped to the last row the workgroup owns.  Later rounds (long lm_heads
+// only) compute their offsets.  Filled once per launch, after the job table.
+__device__ __forceinline__ void build_row_table(const int* table, int* rowtab) {
+  const int i = threadIdx.x;
+  if (i < JK_COUNT * NJMAX) {
+    const int kind = i / NJMAX, e = i - kind * NJMAX;
+    const Job* j = reinterpret_cast<const Job*>(table + kind * NW * 16);  // wave 0's record: these fields are common
+    const int lg = j->bsh - 3;                                            // log2(nrg)
+    const int nbmax = NJMAX >> j->bsh;
+    const int rg = e / (nbmax * RB), b = (e / RB) % nbmax, ii = e % RB;
+    const int njb = j->nj < NJMAX ? j->nj : NJMAX;
+    int row_j = rg + (b << j->bsh) + (ii << lg);
+    row_j = row_j < njb ? row_j : njb - 1;
+    row_j = row_j < 0 ? 0 : row_j;
+    const int row = j->w + j->nwg * (row_j >> j->rsh) + (row_j & ((1 << j->rsh) - 1)) * j->pair_off;
+    rowtab[i] = (int)((unsigned)row * (unsigned)j->K2);
   }
 }
 
@@ -350,8 +378,9 @@ __device__ __forceinline__ Job load_job(const int* table, int kind, int wave, co
   j.K2 = LR_UNI(a.x); j.pair_off = LR_UNI(a.y); j.rsh = LR_UNI(a.z); j.w = LR_UNI(a.w);
   j.nwg = LR_UNI(b.x); j.nj = LR_UNI(b.y); j.ksteps = LR_UNI(b.z); j.nkg = LR_UNI(b.w);
   j.nrg = LR_UNI(c.x); j.rg = LR_UNI(c.y); j.kg = LR_UNI(c.z); j.nk = LR_UNI(c.w);
-  j.bsh = LR_UNI(d.x); j.active = LR_UNI(d.y); j.K = LR_UNI(d.z); j._pad = 0;
+  j.bsh = LR_UNI(d.x); j.active = LR_UNI(d.y); j.K = LR_UNI(d.z); j.kind = kind;
   j.W = W;
+  j.rowtab = table + JK_COUNT * NW * 16 + kind * NJMAX;
   return j;
 }
 
@@ -387,21 +416,32 @@ struct Unit {
 // what lets the compiler's wait-count insertion wait for exactly the older unit (vmcnt(RB))
 // instead of for everything in flight.
 __device__ __forceinline__ void load_unit(const Job& job, int j0, int jb, int kk, int lane, Unit& u, bool real) {
-  const int njb = job.nj - j0 < NJMAX ? job.nj - j0 : NJMAX;
   int k = kk * 512 + lane * 8;
   k = k < job.K ? k : 0;
   const int voff = real ? k * 2 : (int)0x80000000;
-  const int rmask = (1 << job.rsh) - 1;
   __amdgpu_buffer_rsrc_t br = __builtin_amdgcn_make_buffer_rsrc(const_cast<u16*>(job.W), 0, job.W ? 0x7fffffff : 0, 0x00020000);
+  int so[RB];
+  if (j0 == 0) {  // first round: the offsets are tabulated (two LDS reads instead of ~10 scalar operations per row)
+    const int e = ((job.rg * (NJMAX >> job.bsh)) + ((jb - job.rg) >> job.bsh)) * RB;
+    const int4 t0 = *reinterpret_cast<const int4*>(job.rowtab + e);
+    const int4 t1 = *reinterpret_cast<const int4*>(job.rowtab + e + 4);
+    so[0] = t0.x; so[1] = t0.y; so[2] = t0.z; so[3] = t0.w;
+    so[4] = t1.x; so[5] = t1.y; so[6] = t1.z; so[7] = t1.w;
+  } else {
+    const int njb = job.nj - j0 < NJMAX ? job.nj - j0 : NJMAX;
+    const int rmask = (1 << job.rsh) - 1;
 #pragma unroll
-  for (int i = 0; i < RB; ++i) {
-    int j = jb + i * job.nrg;
-    j = j < njb ? j : njb - 1;
-    const int jj = j0 + j;
-    const int row = job.w + job.nwg * (jj >> job.rsh) + (jj & rmask) * job.pair_off;
-    const unsigned soff = real ? (unsigned)row * (unsigned)job.K2 : 0u;
-    u.r[i] = __builtin_amdgcn_raw_buffer_load_b128(br, voff, (int)LR_UNI(soff), 0);
+    for (int i = 0; i < RB; ++i) {
+      int j = jb + i * job.nrg;
+      j = j < njb ? j : njb - 1;
+      const int jj = j0 + j;
+      const int row = job.w + job.nwg * (jj >> job.rsh) + (jj & rmask) * job.pair_off;
+      so[i] = (int)((unsigned)row * (unsigned)job.K2);
+    }
   }
+#pragma unroll
+  for (int i = 0; i < RB; ++i)
+    u.r[i] = __builtin_amdgcn_raw_buffer_load_b128(br, voff, LR_UNI(real ? so[i] : 0), 0);
 }
 // ---- a wave's position in the unit sequence of a job.  The sequence is: for every round, the
 //      wave's units (k-steps fastest, then row batches), padded to an even count, so that the two
@@ -567,7 +607,7 @@ __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, con
         pos_next(job, c);
       }
     }
-    __syncthreads();
+    wg_sync();
     // ---- cross-wave sum in fixed order + epilogue
     const int nout = (njb >> job.rsh) * M;
     if (tid < nout) {
@@ -595,7 +635,7 @@ __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, con
       }
     }
     if (EPI == EPI_LOGITS) {
-      __syncthreads();
+      wg_sync();
       if (tid < M) {  // items ascend with jl: strict '>' keeps the lowest index among equals
         for (int jl = 0; jl < njb; ++jl) {
           const float v = cand_v[jl * M + tid];
@@ -603,7 +643,7 @@ __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, con
         }
       }
     }
-    __syncthreads();
+    wg_sync();
   }
 }
 
@@ -686,7 +726,7 @@ __device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, u1
       red[((tid >> 6) * M + m) * 2 + 1] = ss2[m];
     }
   }
-  __syncthreads();
+  wg_sync();
   // pass 2: scale in place (each lane revisits the elements it wrote)
 #pragma unroll
   for (int m = 0; m < M; ++m) {
@@ -715,7 +755,7 @@ __device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, u1
       }
     }
   }
-  __syncthreads();
+  wg_sync();
 }
 
 // Bring a tagged activation [M][K] into LDS as bf16 (waits for every word).
@@ -727,7 +767,7 @@ __device__ __forceinline__ void load_x(const Coh& coh, unsigned src_wo, unsigned
     coh.ld8(src_wo + c, tag, f);
     st16(x + c, pack8(f));
   }
-  __syncthreads();
+  wg_sync();
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -841,7 +881,7 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
     *reinterpret_cast<u32*>(lp.k_cache + slot) = pack_bf2(r0, r1);
     *reinterpret_cast<u32*>(lp.v_cache + slot) = pack_bf2(v0, v1);
   }
-  __syncthreads();
+  wg_sync();
   if (stamp && tid == 0) stamp[8] = wall_clock64();
   if (n <= 0) {
     for (int i = tid; i < G * HD; i += NT)
@@ -850,7 +890,7 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
       coh.st_f32(ml_out + (unsigned)(tid * NA * 4), -INFINITY, tag);
       coh.st_f32(ml_out + (unsigned)(tid * NA * 4 + 2), 0.0f, tag);
     }
-    __syncthreads();
+    wg_sync();
     return;
   }
   // ---- scores on the matrix cores: S[key][head] = sum_d K[key][d] q[head][d], one 32 x 32 tile per
@@ -884,7 +924,7 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
       }
     }
   }
-  __syncthreads();
+  wg_sync();
   if (stamp && tid == 0) stamp[9] = wall_clock64();
   // ---- softmax statistics: a wave per head; sc becomes exp(s - max)
   for (int g = wave; g < G; g += NW) {
@@ -900,7 +940,7 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
     l = wave_sum(l);
     if (lane == 0) { s_m[g] = m; s_l[g] = l; }
   }
-  __syncthreads();
+  wg_sync();
   if (stamp && tid == 0) stamp[10] = wall_clock64();
   // ---- P.V: GB heads at a time share the unpacked V rows; the key groups of a wave are folded with
   //      lane-half / lane-row swaps (one swap + one add folds two accumulators), the waves in LDS
@@ -951,7 +991,7 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
         *reinterpret_cast<float2*>(ored + (wave * G + g0 + g) * HD + dl + 2 * (lane >> 4)) = make_float2(z0, z1);
     }
   }
-  __syncthreads();
+  wg_sync();
   for (int i = tid; i < G * HD; i += NT) {
     float v = 0.0f;
 #pragma unroll
@@ -962,7 +1002,7 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
     coh.st_f32(ml_out + (unsigned)(tid * NA * 4), s_m[tid], tag);
     coh.st_f32(ml_out + (unsigned)(tid * NA * 4 + 2), s_l[tid], tag);
   }
-  __syncthreads();
+  wg_sync();
 }
 
 // Every workgroup: merge the NA partial attention results into y [M][Hq * HD] (bf16, LDS).
@@ -982,7 +1022,7 @@ __device__ __forceinline__ void attention_merge(const StepParams& p, const Coh& 
     const float L = wave_sum(w * l);
     if (lane < NA) wbuf[bh * NA_MAX + lane] = L > 0.0f ? w / L : 0.0f;
   }
-  __syncthreads();
+  wg_sync();
   for (int pp = tid; pp < npairs; pp += NT) {
     const int bh = (2 * pp) / HD, d = (2 * pp) % HD;
     float y0 = 0.0f, y1 = 0.0f;
@@ -1002,7 +1042,7 @@ __device__ __forceinline__ void attention_merge(const StepParams& p, const Coh& 
     }
     *reinterpret_cast<u32*>(y + 2 * pp) = pack_bf2(y0, y1);
   }
-  __syncthreads();
+  wg_sync();
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1029,7 +1069,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   float* cand_v = wbuf + M * Hq * NA_MAX;               // [NJMAX * M]
   int* cand_i = reinterpret_cast<int*>(cand_v + NJMAX * M);
   int* s_flag = cand_i + NJMAX * M;                     // [8]
-  int* jtab = s_flag + 8;                               // [JK_COUNT][NW][16] job table
+  int* jtab = s_flag + 8;                               // [JK_COUNT][NW][16] job table, then [JK_COUNT][NJMAX] row offsets
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1040,7 +1080,9 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   coh.fail = &ctrl->fail;
   if (tid == 0) s_flag[1] = (int)cldu(&ctrl->epoch_base);
   build_job_table(p, jtab, Hq * HD, w, nwg);
-  __syncthreads();
+  wg_sync();
+  build_row_table(jtab, jtab + JK_COUNT * NW * 16);
+  wg_sync();
   const unsigned epoch_base = (unsigned)s_flag[1];
   int pos = p.pos[0];
   pos = pos < 0 ? 0 : (pos >= p.Smax ? p.Smax - 1 : pos);
@@ -1123,7 +1165,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
     LR_STAMP(7)
     // one workgroup-wide look at the failure flag per slot keeps a broken step from running on
     if (tid == 0) s_flag[0] = (int)cldu(&ctrl->fail);
-    __syncthreads();
+    wg_sync();
     if (s_flag[0]) return;
   }
 #undef LR_JOB
@@ -1159,9 +1201,9 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
         const int oi = __shfl_xor(bi, o, LR_WAVE);
         if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
       }
-      __syncthreads();
+      wg_sync();
       if (lane == 0) { cand_v[wave] = bv; cand_i[wave] = bi; }
-      __syncthreads();
+      wg_sync();
       if (tid == 0) {
         for (int wv = 1; wv < NW; ++wv)
           if (cand_v[wv] > bv || (cand_v[wv] == bv && cand_i[wv] < bi)) { bv = cand_v[wv]; bi = cand_i[wv]; }
@@ -1172,7 +1214,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
         if (p.advance && p.history && slot >= 0 && slot < p.hist_len) p.history[(int64_t)m * p.ld_hist + slot] = bi;
       }
     }
-    __syncthreads();
+    wg_sync();
     if (tid == 0) {
       if (p.advance) p.pos[0] = p.pos[0] + 1;
       cstu(&ctrl->epoch_base, (epoch_base + (unsigned)L + 2u) % 65535u);
@@ -1256,7 +1298,7 @@ template <int M, int HD, int G>
 static size_t lds_bytes(int D, int I, int Hq) {
   const int xlen = M * (D > I ? D : I);
   const size_t fl = (size_t)NW * NJMAX * M + NW * M * 2 + G * HD + (size_t)G * att_capacity(HD) + NW * G * HD +
-                    2 * HD + 2 * G + (size_t)M * Hq * NA_MAX + 2 * NJMAX * M + 8 + JK_COUNT * NW * 16;
+                    2 * HD + 2 * G + (size_t)M * Hq * NA_MAX + 2 * NJMAX * M + 8 + JK_COUNT * NW * 16 + JK_COUNT * NJMAX;
   return ((size_t)xlen * 2 + (size_t)M * D) * sizeof(u16) + fl * sizeof(float) + 16;
 }
 
