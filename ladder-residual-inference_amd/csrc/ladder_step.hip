@@ -292,6 +292,15 @@ __device__ __forceinline__ void reduce8(float* v, float& z0, float& z1) {
 // ------------------------------------------------------------------------------------------------
 #define LR_UNI(x) __builtin_amdgcn_readfirstlane(x)
 
+// The pointer records of the layers around the current one are kept in a small LDS ring (filled
+// one layer ahead of use), so that a job never waits for a scalar load from global memory.
+enum { LP_WQKV = 0, LP_WO, LP_W1, LP_W2, LP_ATTN_NORM, LP_FFN_NORM, LP_K_CACHE, LP_V_CACHE };
+__device__ __forceinline__ const u16* ring_ptr(const u32* lring, int layer, int field) {
+  const u32* e = lring + (layer & 3) * 16 + field * 2;
+  const u32 lo = LR_UNI(e[0]), hi = LR_UNI(e[1]);
+  return reinterpret_cast<const u16*>(((unsigned long long)hi << 32) | lo);
+}
+
 // Everything about a job that does not change from layer to layer (all but the matrix pointer) is
 // worked out once per launch, per job kind and wave, and kept in LDS: the per-layer code then has
 // no divisions and little scalar state (a wave issues at most one instruction every four cycles,
@@ -387,20 +396,22 @@ __device__ __forceinline__ Job load_job(const int* table, int kind, int wave, co
 // The jobs of slot t.  kind: 0 wqkv(t), 1 w1(t-1), 2 wo(t), 3 w2(t-1), 4 lm_head; a slot without
 // that module gets a job that owns no rows.  w1 is dealt to the workgroups that do not run
 // attention in the slot.
-__device__ __forceinline__ Job slot_job(const StepParams& p, const int* table, int kind, int t, int wave) {
+__device__ __forceinline__ Job slot_job(const StepParams& p, const int* table, const u32* lring, int kind, int t,
+                                        int wave) {
   const bool a = t < p.L, b = t >= 1 && t <= p.L;
-  int jk = JK_NONE;
-  const u16* W = nullptr;
-  if (kind == 0 && a) { jk = JK_QKV; W = p.layers[t].wqkv; }
-  if (kind == 1 && b) { jk = a ? JK_W1_SPLIT : JK_W1_ALL; W = p.layers[t - 1].w1; }
-  if (kind == 2 && a) { jk = JK_WO; W = p.layers[t].wo; }
-  if (kind == 3 && b) { jk = JK_W2; W = p.layers[t - 1].w2; }
+  int jk = JK_NONE, layer = 0, field = 0;
+  if (kind == 0 && a) { jk = JK_QKV; layer = t; field = LP_WQKV; }
+  if (kind == 1 && b) { jk = a ? JK_W1_SPLIT : JK_W1_ALL; layer = t - 1; field = LP_W1; }
+  if (kind == 2 && a) { jk = JK_WO; layer = t; field = LP_WO; }
+  if (kind == 3 && b) { jk = JK_W2; layer = t - 1; field = LP_W2; }
+  const u16* W = ring_ptr(lring, layer, field);
+  if (jk == JK_NONE) W = nullptr;
   if (kind == 4) { jk = JK_HEAD; W = p.out_w; }
   return load_job(table, jk, wave, W);
 }
 // first job of slot t + 1
-__device__ __forceinline__ Job next_slot_job(const StepParams& p, const int* table, int t, int wave) {
-  return slot_job(p, table, t + 1 < p.L ? 0 : (t + 1 == p.L ? 1 : 4), t + 1, wave);
+__device__ __forceinline__ Job next_slot_job(const StepParams& p, const int* table, const u32* lring, int t, int wave) {
+  return slot_job(p, table, lring, t + 1 < p.L ? 0 : (t + 1 == p.L ? 1 : 4), t + 1, wave);
 }
 
 struct Unit {
@@ -1069,7 +1080,8 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   float* cand_v = wbuf + M * Hq * NA_MAX;               // [NJMAX * M]
   int* cand_i = reinterpret_cast<int*>(cand_v + NJMAX * M);
   int* s_flag = cand_i + NJMAX * M;                     // [8]
-  int* jtab = s_flag + 8;                               // [JK_COUNT][NW][16] job table, then [JK_COUNT][NJMAX] row offsets
+  u32* lring = reinterpret_cast<u32*>(s_flag + 8);      // [4][16] layer pointer records
+  int* jtab = s_flag + 8 + 64;                               // [JK_COUNT][NW][16] job table, then [JK_COUNT][NJMAX] row offsets
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1080,6 +1092,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   coh.fail = &ctrl->fail;
   if (tid == 0) s_flag[1] = (int)cldu(&ctrl->epoch_base);
   build_job_table(p, jtab, Hq * HD, w, nwg);
+  if (tid < 32 && (tid >> 4) < L) lring[tid] = reinterpret_cast<const u32*>(p.layers)[tid];  // layers 0 and 1
   wg_sync();
   build_row_table(jtab, jtab + JK_COUNT * NW * 16);
   wg_sync();
@@ -1095,22 +1108,24 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
 
   const int qdim = Hq * HD;
   Pipe pipe;
-  prime(slot_job(p, jtab, 0, 0, wave), lane, pipe);
+  prime(slot_job(p, jtab, lring, 0, 0, wave), lane, pipe);
 
 #define LR_STAMP(k)                                                                                  \
   if (p.prof && t >= p.prof_t0 && t < p.prof_t0 + PROF_SLOTS && tid == 0)                            \
     p.prof[((size_t)blockIdx.x * PROF_SLOTS + (t - p.prof_t0)) * PROF_POINTS + (k)] = wall_clock64();
-#define LR_JOB(kind) slot_job(p, jtab, kind, t, wave)
+#define LR_JOB(kind) slot_job(p, jtab, lring, kind, t, wave)
   for (int t = 0; t <= L; ++t) {
     const bool has_a = t < L, has_b = t >= 1;
-    const LayerPtrs* la = p.layers + (has_a ? t : L - 1);
-    const LayerPtrs* lb = p.layers + (has_b ? t - 1 : 0);
+    // request the pointer record of layer t + 2 now; it goes into the ring at the end of the slot
+    u32 ring_next = 0;
+    if (tid < 16 && t + 2 < L) ring_next = reinterpret_cast<const u32*>(p.layers + t + 2)[tid];
     const unsigned tag = tag_of(epoch_base + (unsigned)t + 1u), tag_prev = tag_of(epoch_base + (unsigned)t);
     const unsigned act_wo = p.oact + (unsigned)((t & 1) * M * I);  // activations alternate between two buffers
     LR_STAMP(0)
     // ---------------- v1 = R + m(t-2) feeds mlp(t-1); v2 = v1 + a(t-1) feeds attention(t)
     prologue<M>(p, coh, xr, t == 0 ? p.tokens : nullptr, t >= 2, p.om, tag_prev, t >= 1 && has_a, p.oa, tag_prev,
-                has_b ? lb->ffn_norm : nullptr, has_a ? la->attn_norm : nullptr, xb, xa, red);
+                has_b ? ring_ptr(lring, t - 1, LP_FFN_NORM) : nullptr,
+                has_a ? ring_ptr(lring, t, LP_ATTN_NORM) : nullptr, xb, xa, red);
     // this workgroup no longer reads a / m / the previous partials
     if (tid == 0) coh.st(p.odone + (unsigned)w, 0.0f, tag);
     LR_STAMP(1)
@@ -1120,11 +1135,14 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
       LR_STAMP(2)
       // ---------------- attention workgroup (it owns no rows of w1)
       KV<HD> kv;
+      LayerPtrs lcache;  // only the cache pointers are used
+      lcache.k_cache = const_cast<u16*>(ring_ptr(lring, t, LP_K_CACHE));
+      lcache.v_cache = const_cast<u16*>(ring_ptr(lring, t, LP_V_CACHE));
       bool first = true;
       for (int b = 0; b < p.B; ++b)
         for (int kvh = 0; kvh < p.Hkv; ++kvh) {
-          attention_load<HD>(p, *la, b, kvh, k0, k1, pos, kv);
-          attention_compute<M, HD, G>(p, coh, *la, b, kvh, k0, k1, pos, tag, first,
+          attention_load<HD>(p, lcache, b, kvh, k0, k1, pos, kv);
+          attention_compute<M, HD, G>(p, coh, lcache, b, kvh, k0, k1, pos, tag, first,
                                       (p.prof && t >= p.prof_t0 && t < p.prof_t0 + PROF_SLOTS)
                                           ? p.prof + ((size_t)blockIdx.x * PROF_SLOTS + (t - p.prof_t0)) * PROF_POINTS
                                           : nullptr,
@@ -1145,7 +1163,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
     if (has_a) {
       attention_merge<M, HD>(p, coh, Hq, tag, xa, wbuf);
       LR_STAMP(4)
-      Job after_wo = next_slot_job(p, jtab, t, wave);
+      Job after_wo = next_slot_job(p, jtab, lring, t, wave);
       if (has_b) after_wo = LR_JOB(3);
       run_job<M, EPI_STORE>(p, coh, LR_JOB(2), after_wo, pipe, xa, part, p.oa, D, tag, nullptr, nullptr, nullptr,
                             nullptr);
@@ -1159,10 +1177,11 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
     if (has_b) {
       load_x<M>(coh, act_wo, tag, I, xb);
       LR_STAMP(6)
-      run_job<M, EPI_STORE>(p, coh, LR_JOB(3), next_slot_job(p, jtab, t, wave), pipe, xb, part, p.om, D, tag,
+      run_job<M, EPI_STORE>(p, coh, LR_JOB(3), next_slot_job(p, jtab, lring, t, wave), pipe, xb, part, p.om, D, tag,
                             nullptr, nullptr, nullptr, nullptr);
     }
     LR_STAMP(7)
+    if (tid < 16 && t + 2 < L) lring[((t + 2) & 3) * 16 + tid] = ring_next;
     // one workgroup-wide look at the failure flag per slot keeps a broken step from running on
     if (tid == 0) s_flag[0] = (int)cldu(&ctrl->fail);
     wg_sync();
@@ -1176,7 +1195,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
               p.final_norm, xb, xa, red);
   float best_v = -INFINITY;
   int best_i = 0x7fffffff;
-  run_job<M, EPI_LOGITS>(p, coh, slot_job(p, jtab, 4, L + 1, wave), slot_job(p, jtab, -1, 0, wave), pipe,
+  run_job<M, EPI_LOGITS>(p, coh, slot_job(p, jtab, lring, 4, L + 1, wave), slot_job(p, jtab, lring, -1, 0, wave), pipe,
                          xa, part, 0u, 0, tag,
                          cand_v, cand_i, &best_v, &best_i);
   if (tid < M) {  // candidate: value (bf16-exact), a filler word, index as two 16-bit halves
@@ -1298,7 +1317,7 @@ template <int M, int HD, int G>
 static size_t lds_bytes(int D, int I, int Hq) {
   const int xlen = M * (D > I ? D : I);
   const size_t fl = (size_t)NW * NJMAX * M + NW * M * 2 + G * HD + (size_t)G * att_capacity(HD) + NW * G * HD +
-                    2 * HD + 2 * G + (size_t)M * Hq * NA_MAX + 2 * NJMAX * M + 8 + JK_COUNT * NW * 16 + JK_COUNT * NJMAX;
+                    2 * HD + 2 * G + (size_t)M * Hq * NA_MAX + 2 * NJMAX * M + 8 + 64 + JK_COUNT * NW * 16 + JK_COUNT * NJMAX;
   return ((size_t)xlen * 2 + (size_t)M * D) * sizeof(u16) + fl * sizeof(float) + 16;
 }
 
