@@ -1275,7 +1275,13 @@ int g_na_override = -1;  // tuning hook: number of attention workgroups (must st
 static int pick_na(int Smax, int hd, int nwg) {
   const int cap = att_capacity(hd);
   int na = (Smax + cap - 1) / cap;
-  if (g_na_override > na) na = g_na_override;
+  // more attention workgroups than capacity requires pay off up to about 128 keys each: attention is
+  // instruction bound and sits on the critical path next to the w1 stream
+  int want = (Smax + 127) / 128;
+  if (want > NA_MAX) want = NA_MAX;
+  if (want > nwg / 8) want = nwg / 8;
+  if (want > na) na = want;
+  if (g_na_override > 0) na = g_na_override > na ? g_na_override : na;
   if (na < 1) na = 1;
   if (na >= nwg) na = nwg - 1;
   return na;
