@@ -674,6 +674,14 @@ __device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, u1
                                          unsigned d2_tag, const u16* g1, const u16* g2, u16* x1, u16* x2, float* red) {
   const int tid = opaque_tid(), D = p.D;
   float ss1[M], ss2[M];
+  // the gains are needed only in pass 2 but are requested now: their latency hides behind pass 1
+  uint4 gq1[PRO_NIT], gq2[PRO_NIT];
+#pragma unroll
+  for (int it = 0; it < PRO_NIT; ++it) {
+    const int c = (it * NT + tid) * 8;
+    gq1[it] = (g1 && c < D) ? ld16(g1 + c) : make_uint4(0, 0, 0, 0);
+    gq2[it] = (g2 && c < D) ? ld16(g2 + c) : make_uint4(0, 0, 0, 0);
+  }
   // pass 1: the (bf16-exact) sums go to LDS unscaled; sums of squares per lane
 #pragma unroll
   for (int m = 0; m < M; ++m) {
@@ -748,18 +756,21 @@ __device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, u1
       s2 += red[(wv * M + m) * 2 + 1];
     }
     const float inv1 = rsqrtf(s1 / (float)D + p.eps), inv2 = rsqrtf(s2 / (float)D + p.eps);
-    for (int c = tid * 8; c < D; c += NT * 8) {
+#pragma unroll
+    for (int it = 0; it < PRO_NIT; ++it) {
+      const int c = (it * NT + tid) * 8;
+      if (c >= D) break;
       float v[8], g[8], o[8];
       if (g1) {
         unpack8(*reinterpret_cast<const uint4*>(x1 + m * D + c), v);
-        unpack8(ld16(g1 + c), g);
+        unpack8(gq1[it], g);
 #pragma unroll
         for (int j = 0; j < 8; ++j) o[j] = round_bf(v[j] * inv1) * g[j];
         st16(x1 + m * D + c, pack8(o));
       }
       if (g2) {
         unpack8(*reinterpret_cast<const uint4*>(x2 + m * D + c), v);
-        unpack8(ld16(g2 + c), g);
+        unpack8(gq2[it], g);
 #pragma unroll
         for (int j = 0; j < 8; ++j) o[j] = round_bf(v[j] * inv2) * g[j];
         st16(x2 + m * D + c, pack8(o));
@@ -1024,6 +1035,15 @@ __device__ __forceinline__ void attention_merge(const StepParams& p, const Coh& 
   const int tid = opaque_tid(), wave = tid >> 6, lane = tid & 63;
   const int NA = p.NA, nbh = p.B * Hq;
   const int npairs = nbh * HD / 2;
+  // the partial outputs of this lane's first pair are requested before the weights are worked out
+  u32x4_t raw[NA_MAX];
+  {
+    const int bh = (2 * tid) / HD, d = (2 * tid) % HD;
+#pragma unroll
+    for (int s = 0; s < NA_MAX; ++s)
+      raw[s] = (s < NA && tid < npairs) ? coh.raw4(p.oopart + (unsigned)(((bh * NA + s) * HD + d) * 2))
+                                        : u32x4_t{0u, 0u, 0u, 0u};
+  }
   // weights: a wave per (sequence, head); lanes < NA hold one chunk each
   for (int bh = wave; bh < nbh; bh += NW) {
     float m = -INFINITY, l = 0.0f;
@@ -1037,10 +1057,11 @@ __device__ __forceinline__ void attention_merge(const StepParams& p, const Coh& 
   for (int pp = tid; pp < npairs; pp += NT) {
     const int bh = (2 * pp) / HD, d = (2 * pp) % HD;
     float y0 = 0.0f, y1 = 0.0f;
-    u32x4_t raw[NA_MAX];
+    if (pp != tid) {
 #pragma unroll
-    for (int s = 0; s < NA_MAX; ++s)
-      if (s < NA) raw[s] = coh.raw4(p.oopart + (unsigned)(((bh * NA + s) * HD + d) * 2));
+      for (int s = 0; s < NA_MAX; ++s)
+        if (s < NA) raw[s] = coh.raw4(p.oopart + (unsigned)(((bh * NA + s) * HD + d) * 2));
+    }
 #pragma unroll
     for (int s = 0; s < NA_MAX; ++s) {
       if (s < NA) {
