@@ -12,9 +12,10 @@
 //     residual adds + both RMSNorms (redundantly in every workgroup; the residual stream itself
 //         never leaves the workgroup's LDS)
 //     wqkv(t) rows
-//     attention workgroups (a handful): attention(t) over their key range with K/V held in
-//         registers, un-normalised partial results
-//     all other workgroups: w1(t-1) rows + SwiGLU  (18 us of streaming that hides the attention
+//     attention workgroups (about one per 128 keys): attention(t) over their key range with K/V
+//         held in registers -- scores on the matrix cores (v_mfma_f32_32x32x16_bf16, one tile per
+//         32 keys), fp32 softmax and P.V -- un-normalised partial results
+//     all other workgroups: w1(t-1) rows + SwiGLU  (17 us of streaming that hides the attention
 //         latency chain)
 //     merge the partial results, wo(t) rows
 //     w2(t-1) rows
@@ -34,13 +35,24 @@
 // rounds (fp32 attention partials take two words).  Weights, KV cache and logits use ordinary
 // accesses (read-only, or produced for the next launch).
 //
-// Weight streaming never stops at these edges: every wave walks its GEMV work of the whole slot
-// (and the first job of the next one) as a sequence of "units" (8 rows x 1 KiB of one K-slice)
-// through a prefetch cursor that runs two units ahead of the multiplier, across job boundaries,
-// reductions, epilogues, norms and waits, so each wave keeps 16 KiB of loads in flight.  GEMV
+// Weight streaming does not stop at these edges: every wave walks its GEMV work as a sequence of
+// "units" (8 rows x 1 KiB of one K-slice) held in two register sets; the set just multiplied is
+// refilled at once with the unit two positions ahead -- also across the end of a job into the
+// next one, through reductions, epilogues, norms and waits -- so a wave has 16 KiB of loads in
+// flight.  The unit sequence of a job is padded to an even length (pad loads go out of the
+// buffer's range and cost nothing) so that the two sets alternate in a fixed pattern, there is
+// exactly ONE load sequence in the loop, and rows are addressed through a scalar offset from a
+// small per-launch table: that is what lets the compiler place exact wait counts (vmcnt(8))
+// instead of draining the pipeline.  The multiply is v_dot2_f32_bf16 on packed bf16 pairs.  GEMV
 // rows are dealt to workgroups round-robin so that the CUs working at the same time read
 // neighbouring rows (HBM-channel friendly); inside a workgroup the waves split K, partial sums
-// meet in LDS in a fixed order -- no float atomics, bit-reproducible.
+// meet in LDS in a fixed order -- no float atomics, bit-reproducible.  Workgroup barriers wait for
+// LDS only (wg_sync): __syncthreads() would also wait for the prefetched units.
+//
+// A wave issues at most one instruction every four cycles, so bookkeeping is kept off the layer
+// loop: everything about a job except its matrix pointer is tabulated once per launch in LDS
+// (per job kind and wave), row offsets included, and the pointer records of the neighbouring
+// layers sit in a small LDS ring filled one layer ahead.
 //
 // Every retry loop is bounded: on time-out a workgroup raises ctrl->fail and goes on with
 // whatever it has; everybody leaves at the end of the slot in which they see the flag, so the
