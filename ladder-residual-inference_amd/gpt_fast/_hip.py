@@ -150,6 +150,19 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, act_swiglu: bool
     return out
 
 
+def linear_swiglu(h: torch.Tensor, w: torch.Tensor, out: torch.Tensor, act: torch.Tensor = None):
+    """out = (silu(g) * u) @ w^T for h = [u | g].  Up to 8 rows the activation is fused into the
+    weight-streaming GEMV; above that it is materialised once (in `act`, or a new tensor) and fed to
+    the plain MFMA GEMM, whose operand loader is then a pure copy."""
+    M, two_k, _ = _rows_ld(h)
+    if M <= 8:
+        return linear(h, w, out, act_swiglu=True)
+    if act is None:
+        act = h.new_empty(M, two_k // 2)
+    swiglu(h, act)
+    return linear(act, w, out)
+
+
 def swiglu(h: torch.Tensor, out: torch.Tensor):
     rows, two_i, ldh = _rows_ld(h)
     assert out.is_contiguous() and out.numel() == rows * (two_i // 2)

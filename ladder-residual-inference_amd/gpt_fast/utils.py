@@ -130,7 +130,7 @@ class FeedForward(nn.Module):
         x = x.contiguous()
         lead = x.shape[:-1]
         h = _hip.linear(x, self.w1.weight, x.new_empty(*lead, self.w1.out_features))
-        return _hip.linear(h, self.w2.weight, x.new_empty(*lead, self.w2.out_features), act_swiglu=True)
+        return _hip.linear_swiglu(h, self.w2.weight, x.new_empty(*lead, self.w2.out_features))
 
 
 class _AttentionCore(nn.Module):
@@ -224,6 +224,5 @@ class FuseAttentionMLP(_AttentionCore):
         fused = _hip.linear(x, self.wqkv1.weight, x.new_empty(bsz, seqlen, self.wqkv1.out_features))
         y = self._attend(fused, bsz, seqlen, freqs_cis, input_pos)
         a = _hip.linear(y, self.wo.weight, x.new_empty(bsz, seqlen, self.wo.out_features))
-        m = _hip.linear(fused[..., nqkv:], self.w2.weight, x.new_empty(bsz, seqlen, self.w2.out_features),
-                        act_swiglu=True)
+        m = _hip.linear_swiglu(fused[..., nqkv:], self.w2.weight, x.new_empty(bsz, seqlen, self.w2.out_features))
         return _hip.add(m, a, m)
