@@ -341,6 +341,192 @@ __global__ __launch_bounds__(64) void k_attn_prefill(const u16* __restrict__ q, 
   }
 }
 
+// ----------------------------------------------------------------------- prefill on the matrix cores
+// Flash-style causal attention in the TRANSPOSED form, so that everything per query sits in one lane:
+//   S^T[key][q]  = sum_d K[key][d] Q[q][d]          (A = K tile from LDS, B = Q from registers)
+//   O^T[d][q]   += sum_key V^T[d][key] P^T[key][q]  (A = V^T tile from LDS, B = P^T from the S^T registers)
+// with v_mfma_f32_32x32x16_bf16.  An accumulator column is a query (lane % 32), so row maxima, sums and
+// the rescaling factor are per-lane scalars; the 16 S^T values a lane holds for its query are exactly,
+// in order, the B operand of the two PV k-steps (the key order of a k-step is free as long as the V^T
+// operand uses the same one), so P never moves between lanes.  P enters the bf16 MFMA as hi + lo
+// (p = bf16(p) + bf16(p - bf16(p))), which keeps the fp32 softmax weights to ~2^-17: the result matches
+// the fp32 "math" attention of the eager reference (utils.py:247-258) to rounding of the final bf16.
+// A workgroup is 4 waves = NWH heads of one kv head x NWQ tiles of 32 queries sharing the K / V tiles.
+template <int HD, int NWH>
+__global__ __launch_bounds__(256) void k_attn_prefill_mfma(const u16* __restrict__ q, int64_t ldq,
+                                                           const u16* __restrict__ kc, const u16* __restrict__ vc,
+                                                           const int32_t* __restrict__ pos, u16* __restrict__ y,
+                                                           int64_t ldy, int S, int Hq, int Hkv, int Smax) {
+  constexpr int NWQ = 4 / NWH;            // query tiles per workgroup
+  constexpr int KS = HD / 16;             // k-steps of the score product
+  constexpr int DT = HD / 32;             // 32-row tiles of O^T
+  constexpr int KROW = HD + 8;            // K tile row length in elements (16 B pad: conflict-free 128-bit reads)
+  constexpr int VROW = 32 + 4;            // V^T tile row length in elements (8 B pad)
+  __shared__ __attribute__((aligned(16))) u16 ks[32 * KROW];
+  __shared__ __attribute__((aligned(16))) u16 vt[HD * VROW];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int col = lane & 31, half = lane >> 5;
+  const int G = Hq / Hkv;
+  const int hgroups = G / NWH;                       // workgroups per kv head along heads
+  const int kvh = blockIdx.y / hgroups;
+  const int head = kvh * G + (blockIdx.y % hgroups) * NWH + (wave % NWH);
+  const int b = blockIdx.z;
+  const int s = (blockIdx.x * NWQ + wave / NWH) * 32 + col;  // this lane's query
+  const bool valid = s < S;
+  int p = valid ? pos[s] : -1;
+  p = p >= Smax ? Smax - 1 : p;
+  // keys needed by anybody in the workgroup
+  int kmax = p;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const int t = __shfl_xor(kmax, o, LR_WAVE);
+    kmax = t > kmax ? t : kmax;
+  }
+  __shared__ int s_kmax[4];
+  if (lane == 0) s_kmax[wave] = kmax;
+  __syncthreads();
+  kmax = max(max(s_kmax[0], s_kmax[1]), max(s_kmax[2], s_kmax[3]));
+  const int nkeys = kmax + 1;
+
+  // Q as B operands: k-step ks_ holds elements 16 ks_ + 8 half .. + 8 of this lane's query
+  u32x4_t qb[KS];
+  {
+    const u16* qrow = q + ((int64_t)b * S + (valid ? s : 0)) * ldq + head * HD;
+#pragma unroll
+    for (int i = 0; i < KS; ++i) {
+      const uint4 t = valid ? ld16(qrow + 16 * i + 8 * half) : make_uint4(0, 0, 0, 0);
+      qb[i] = u32x4_t{t.x, t.y, t.z, t.w};
+    }
+  }
+  f32x16_t o[DT];
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[d][v] = 0.0f;
+  float m = -INFINITY, l = 0.0f;  // l: this lane's half of the row sum
+  const float scale = rsqrtf((float)HD);
+  const u16* kbase = kc + ((int64_t)b * Hkv + kvh) * Smax * HD;
+  const u16* vbase = vc + ((int64_t)b * Hkv + kvh) * Smax * HD;
+
+  for (int t0 = 0; t0 < nkeys; t0 += 32) {
+    __syncthreads();
+    // ---- stage 32 keys: K row-major, V transposed ([d][key])
+    for (int c = tid; c < 32 * HD / 8; c += 256) {
+      const int key = c / (HD / 8), d = (c % (HD / 8)) * 8;
+      uint4 kk = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
+      if (t0 + key < nkeys) {
+        kk = ld16(kbase + (int64_t)(t0 + key) * HD + d);
+        vv = ld16(vbase + (int64_t)(t0 + key) * HD + d);
+      }
+      *reinterpret_cast<uint4*>(&ks[key * KROW + d]) = kk;
+      const u32 w4[4] = {vv.x, vv.y, vv.z, vv.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        vt[(d + 2 * j) * VROW + key] = (u16)(w4[j] & 0xffffu);
+        vt[(d + 2 * j + 1) * VROW + key] = (u16)(w4[j] >> 16);
+      }
+    }
+    __syncthreads();
+    // ---- S^T tile: rows = keys, columns = queries
+    f32x16_t sacc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) sacc[v] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < KS; ++i) {
+      const uint4 t = *reinterpret_cast<const uint4*>(&ks[col * KROW + 16 * i + 8 * half]);
+      const u32x4_t ka = {t.x, t.y, t.z, t.w};
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, ka), __builtin_bit_cast(bf16x8_t, qb[i]),
+                                                     sacc, 0, 0, 0);
+    }
+    // element v is key t0 + (v / 4) * 8 + half * 4 + v % 4 for query `col`
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int key = t0 + (v / 4) * 8 + half * 4 + (v % 4);
+      sacc[v] = key <= p ? sacc[v] * scale : -INFINITY;
+      tmax = fmaxf(tmax, sacc[v]);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, LR_WAVE));
+    const float mn = fmaxf(m, tmax);
+    float corr = 1.0f;
+    u32x4_t phi[2], plo[2];
+    if (mn != -INFINITY) {
+      corr = expf(m - mn);  // m == -inf -> 0
+      l *= corr;
+      float pv[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        pv[v] = expf(sacc[v] - mn);  // masked -> 0
+        l += pv[v];
+      }
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2) {
+        u32 hi[4], lo[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float a0 = pv[8 * h2 + 2 * j], a1 = pv[8 * h2 + 2 * j + 1];
+          const float h0 = round_bf(a0), h1 = round_bf(a1);
+          hi[j] = pack_bf2(h0, h1);
+          lo[j] = pack_bf2(a0 - h0, a1 - h1);
+        }
+        phi[h2] = u32x4_t{hi[0], hi[1], hi[2], hi[3]};
+        plo[h2] = u32x4_t{lo[0], lo[1], lo[2], lo[3]};
+      }
+      m = mn;
+    } else {
+      phi[0] = phi[1] = plo[0] = plo[1] = u32x4_t{0u, 0u, 0u, 0u};
+    }
+    // ---- O^T += V^T P^T ; k-step h2 covers keys 16 h2 + {0..3, 8..11} + 4 half, in the order of sacc
+#pragma unroll
+    for (int d = 0; d < DT; ++d) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o[d][v] *= corr;
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2) {
+        const u16* vr = &vt[(d * 32 + col) * VROW + 16 * h2 + 4 * half];
+        const uint2 v0 = *reinterpret_cast<const uint2*>(vr), v1 = *reinterpret_cast<const uint2*>(vr + 8);
+        const u32x4_t va = {v0.x, v0.y, v1.x, v1.y};
+        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, va), __builtin_bit_cast(bf16x8_t, phi[h2]),
+                                                       o[d], 0, 0, 0);
+        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, va), __builtin_bit_cast(bf16x8_t, plo[h2]),
+                                                       o[d], 0, 0, 0);
+      }
+    }
+  }
+  l += __shfl_xor(l, 32, LR_WAVE);
+  if (valid) {
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    u16* yrow = y + ((int64_t)b * S + s) * ldy + head * HD;
+    // element v of tile d: dimension d * 32 + (v / 4) * 8 + half * 4 + v % 4
+#pragma unroll
+    for (int d = 0; d < DT; ++d)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        uint2 w2;
+        w2.x = pack_bf2(o[d][4 * g4] * inv, o[d][4 * g4 + 1] * inv);
+        w2.y = pack_bf2(o[d][4 * g4 + 2] * inv, o[d][4 * g4 + 3] * inv);
+        *reinterpret_cast<uint2*>(yrow + d * 32 + g4 * 8 + half * 4) = w2;
+      }
+  }
+}
+
+template <int HD>
+static int launch_prefill_mfma(const u16* q, int64_t ldq, const u16* kc, const u16* vc, const int32_t* pos, u16* y,
+                               int64_t ldy, int B, int S, int Hq, int Hkv, int Smax, hipStream_t s) {
+  const int G = Hq / Hkv;
+  if (G % 4 == 0) {
+    k_attn_prefill_mfma<HD, 4><<<dim3((S + 31) / 32, Hq / 4, B), dim3(256), 0, s>>>(q, ldq, kc, vc, pos, y, ldy, S, Hq,
+                                                                                  Hkv, Smax);
+  } else if (G % 2 == 0) {
+    k_attn_prefill_mfma<HD, 2><<<dim3((S + 63) / 64, Hq / 2, B), dim3(256), 0, s>>>(q, ldq, kc, vc, pos, y, ldy, S, Hq,
+                                                                                  Hkv, Smax);
+  } else {
+    k_attn_prefill_mfma<HD, 1><<<dim3((S + 127) / 128, Hq, B), dim3(256), 0, s>>>(q, ldq, kc, vc, pos, y, ldy, S, Hq,
+                                                                                Hkv, Smax);
+  }
+  return lr_launch_status();
+}
+
 extern "C" int lr_attn_prefill(const void* q, int64_t ldq, const void* k_cache, const void* v_cache,
                                const int32_t* pos, void* y, int64_t ldy, int B, int S, int Hq, int Hkv, int hd,
                                int Smax, lr_stream_t stream) {
@@ -354,6 +540,14 @@ extern "C" int lr_attn_prefill(const void* q, int64_t ldq, const void* k_cache, 
   if (ldq % 8 || ldy % 8) return LR_E_ALIGN;
   const dim3 grid((S + 63) / 64, Hq, B);
   hipStream_t s = (hipStream_t)stream;
+  if (S >= 16 && Hq <= 65535 * 4) {  // matrix-core kernel; the lane-per-query kernel below serves short inputs
+    if (hd == 128)
+      return launch_prefill_mfma<128>((const u16*)q, ldq, (const u16*)k_cache, (const u16*)v_cache, pos, (u16*)y, ldy,
+                                      B, S, Hq, Hkv, Smax, s);
+    if (hd == 64)
+      return launch_prefill_mfma<64>((const u16*)q, ldq, (const u16*)k_cache, (const u16*)v_cache, pos, (u16*)y, ldy, B,
+                                     S, Hq, Hkv, Smax, s);
+  }
   if (hd == 128)
     k_attn_prefill<128><<<grid, dim3(64), 0, s>>>((const u16*)q, ldq, (const u16*)k_cache, (const u16*)v_cache, pos,
                                                   (u16*)y, ldy, S, Hq, Hkv, Smax);

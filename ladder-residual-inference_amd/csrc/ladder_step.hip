@@ -101,8 +101,6 @@ struct StepParams {
   int prof_t0;
 };
 
-typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
 
 // The lane index as a value the optimiser cannot see through: index arithmetic derived from it
 // stays inside the phase that uses it instead of being hoisted out of the layer loop (where it

@@ -257,6 +257,10 @@ def test_attn_decode(hip, B, Hq, Hkv, hd, Smax, pos):
 @pytest.mark.parametrize("B,S,Hq,Hkv,hd,Smax,start", [
     (1, 128, 8, 1, 128, 136, 0), (2, 100, 4, 2, 64, 160, 0), (1, 300, 8, 1, 128, 512, 100), (1, 2048, 8, 1, 128, 2176, 0),
     (3, 65, 32, 8, 64, 72, 0),
+    # one q head per kv head (4 query tiles per workgroup), odd group sizes, 16 heads per kv head, S below the
+    # matrix-core kernel's threshold, a single query tile with a long history
+    (2, 130, 4, 4, 128, 136, 0), (1, 97, 6, 2, 64, 104, 3), (1, 64, 16, 1, 128, 64, 0), (2, 9, 8, 2, 64, 16, 0),
+    (1, 17, 8, 1, 128, 1024, 1000),
 ])
 def test_attn_prefill(hip, B, S, Hq, Hkv, hd, Smax, start):
     q = rnd(B, S, Hq * hd, seed=24)
