@@ -123,6 +123,118 @@ __global__ __launch_bounds__(256) void k_gemm(const u16* __restrict__ x, int64_t
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Skinny GEMM for decode batches (4 < M <= 64): the weights are streamed once, the few input rows
+// ride along.  A workgroup owns 32 weight rows (N / 32 workgroups: every CU has work even for the
+// 1280-row wqkv), stages [32 x 128] weight and [MT x 128] input tiles through LDS (coalesced
+// 16-byte loads, double buffered) and its 4 waves split the tile's 8 k-steps; their partial
+// accumulators meet in LDS at the end.  y^T = W x^T on the matrix cores: A = weight rows,
+// B = input rows (MT / 32 column tiles), so a lane ends up with 4 consecutive n of one m.
+// ---------------------------------------------------------------------------------------------
+constexpr int SN = 32, SK = 128, SLD = SK + 8;
+
+template <int MT>
+__global__ __launch_bounds__(256) void k_gemm_skinny(const u16* __restrict__ x, int64_t ldx, const u16* __restrict__ w,
+                                                     u16* __restrict__ y, int64_t ldy, int M, int N, int K) {
+  constexpr int CT = MT / 32;                       // column tiles (input rows / 32)
+  constexpr int XCH = MT * SK / 8 / 256;            // 16-byte chunks of the input tile per thread
+  constexpr int WCH = SN * SK / 8 / 256;            // ... of the weight tile
+  constexpr int STAGE = (SN + MT) * SLD;            // elements per LDS stage
+  constexpr int LDS_ELEMS = 2 * STAGE > 4 * CT * 16 * 64 * 2 ? 2 * STAGE : 4 * CT * 16 * 64 * 2;
+  __shared__ __attribute__((aligned(16))) u16 lds[LDS_ELEMS];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n0 = blockIdx.x * SN;
+  const int arow = lane & 31, akq = (lane >> 5) * 8;
+
+  f32x16_t acc[CT];
+#pragma unroll
+  for (int c = 0; c < CT; ++c)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[c][v] = 0.0f;
+
+  uint4 xr[XCH], wr[WCH];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < WCH; ++i) {
+      const int id = tid + i * 256, r = id >> 4, c = (id & 15) * 8;
+      wr[i] = load_w_chunk(w, N, K, n0 + r, k0 + c);
+    }
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) {
+      const int id = tid + i * 256, r = id >> 4, c = (id & 15) * 8;
+      xr[i] = load_x_chunk<false>(x, ldx, M, K, r, k0 + c);
+    }
+  };
+  auto stage = [&](int buf) {
+    u16* ws_ = lds + buf * STAGE;
+    u16* xs_ = ws_ + SN * SLD;
+#pragma unroll
+    for (int i = 0; i < WCH; ++i) {
+      const int id = tid + i * 256, r = id >> 4, c = (id & 15) * 8;
+      st16(&ws_[r * SLD + c], wr[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) {
+      const int id = tid + i * 256, r = id >> 4, c = (id & 15) * 8;
+      st16(&xs_[r * SLD + c], xr[i]);
+    }
+  };
+  const int nk = (K + SK - 1) / SK;
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  for (int kt = 0; kt < nk; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < nk) fetch((kt + 1) * SK);
+    const u16* ws_ = lds + cur * STAGE;
+    const u16* xs_ = ws_ + SN * SLD;
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {  // this wave's two k-steps of the tile
+      const int kk = (wave * 2 + q) * 16;
+      const bf16x8_t af = *reinterpret_cast<const bf16x8_t*>(&ws_[arow * SLD + kk + akq]);
+#pragma unroll
+      for (int c = 0; c < CT; ++c) {
+        const bf16x8_t bfr = *reinterpret_cast<const bf16x8_t*>(&xs_[(c * 32 + arow) * SLD + kk + akq]);
+        acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bfr, acc[c], 0, 0, 0);
+      }
+    }
+    if (kt + 1 < nk) stage(cur ^ 1);
+    __syncthreads();
+  }
+  // ---- sum the four waves' partial accumulators in a fixed order
+  float* red = reinterpret_cast<float*>(lds);  // [wave][c][v][lane]
+#pragma unroll
+  for (int c = 0; c < CT; ++c)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) red[((wave * CT + c) * 16 + v) * 64 + lane] = acc[c][v];
+  __syncthreads();
+  // wave w finishes accumulator elements v = 4 w .. 4 w + 3: four consecutive n of one m per lane
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+    float o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int v = wave * 4 + j;
+      o[j] = (red[((0 * CT + c) * 16 + v) * 64 + lane] + red[((1 * CT + c) * 16 + v) * 64 + lane]) +
+             (red[((2 * CT + c) * 16 + v) * 64 + lane] + red[((3 * CT + c) * 16 + v) * 64 + lane]);
+    }
+    // element v: n = n0 + (v / 4) * 8 + (lane / 32) * 4 + v % 4,  m = c * 32 + lane % 32
+    const int m = c * 32 + (lane & 31), n = n0 + wave * 8 + (lane >> 5) * 4;
+    if (m < M) {
+      if (n + 3 < N) {
+        uint2 pk;
+        pk.x = pack_bf2(o[0], o[1]);
+        pk.y = pack_bf2(o[2], o[3]);
+        *reinterpret_cast<uint2*>(y + (int64_t)m * ldy + n) = pk;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (n + j < N) y[(int64_t)m * ldy + n + j] = f_to_bf(o[j]);
+      }
+    }
+  }
+}
+
 extern "C" int lr_linear(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
                          int act_swiglu, lr_stream_t stream) {
   LR_REQUIRE_PTR(x);
@@ -132,7 +244,15 @@ extern "C" int lr_linear(const void* x, int64_t ldx, const void* w, void* y, int
   if (ldx < (act_swiglu ? 2 : 1) * (int64_t)K || ldy < N) return LR_E_SHAPE;
   if (K % 8 || ldx % 8) return LR_E_ALIGN;
   hipStream_t s = (hipStream_t)stream;
-  if (M <= 8) return lr_gemv_dispatch(x, ldx, w, y, ldy, M, N, K, act_swiglu, s);
+  if (M <= 4 || (act_swiglu && M <= 8)) return lr_gemv_dispatch(x, ldx, w, y, ldy, M, N, K, act_swiglu, s);
+  if (!act_swiglu && M <= 64 && ldy % 4 == 0) {
+    const dim3 sgrid((N + SN - 1) / SN);
+    if (M <= 32)
+      k_gemm_skinny<32><<<sgrid, dim3(256), 0, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy, M, N, K);
+    else
+      k_gemm_skinny<64><<<sgrid, dim3(256), 0, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy, M, N, K);
+    return lr_launch_status();
+  }
   const dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
   if (grid.y > 65535) return LR_E_UNSUPPORTED;
   if (act_swiglu)

@@ -151,11 +151,11 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, act_swiglu: bool
 
 
 def linear_swiglu(h: torch.Tensor, w: torch.Tensor, out: torch.Tensor, act: torch.Tensor = None):
-    """out = (silu(g) * u) @ w^T for h = [u | g].  Up to 8 rows the activation is fused into the
+    """out = (silu(g) * u) @ w^T for h = [u | g].  Up to 4 rows the activation is fused into the
     weight-streaming GEMV; above that it is materialised once (in `act`, or a new tensor) and fed to
     the plain MFMA GEMM, whose operand loader is then a pure copy."""
     M, two_k, _ = _rows_ld(h)
-    if M <= 8:
+    if M <= 4:
         return linear(h, w, out, act_swiglu=True)
     if act is None:
         act = h.new_empty(M, two_k // 2)

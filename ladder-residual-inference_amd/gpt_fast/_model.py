@@ -33,7 +33,7 @@ class Workspace:
         self.qkv = e(rows, fused_width)
         self.y = e(rows, cfg.n_head_local * hd)
         self.h = e(rows, 2 * cfg.ffn_local)
-        self.act = e(rows, cfg.ffn_local) if rows > 8 else None   # activated MLP input for the GEMM path
+        self.act = e(rows, cfg.ffn_local) if rows > 4 else None   # activated MLP input for the GEMM path
         self.logits = e(B, S if all_logits else 1, cfg.output_rows)
         self.next_token = torch.empty(B, 1, dtype=torch.int32, device=device)
         self.next_token_valid_for = None   # set by a fused decode step that already chose the token

@@ -145,6 +145,25 @@ def test_linear_gemv(hip, M, N, K):
     assert_close_ulp(y, F.linear(x, w), max_frac=0.05, what="gemv vs F.linear")
 
 
+@pytest.mark.parametrize("N,K", [(1280, 8192), (7168, 8192), (8192, 3584), (16032, 8192), (4096, 4096), (24, 64),
+                                 (1001, 520), (130, 136)])
+@pytest.mark.parametrize("M", [5, 8, 16, 31, 33, 64])
+def test_linear_skinny_batches(hip, M, N, K):
+    """Decode batches (4 < M <= 64) take the skinny matrix-core GEMM: ragged N, K not a multiple of the
+    128-element tile, M on both sides of the 32-row column tile, a strided output view."""
+    if M in (31, 33) and N * K > 20e6:
+        pytest.skip("odd batch sizes are covered on the smaller shapes")
+    x = rnd(M, K, seed=12)
+    w = rnd(N, K, seed=13, scale=0.02)
+    y = torch.empty(M, N, dtype=BF, device=DEV)
+    hip.linear(x, w, y)
+    assert_close_ulp(y, linear_ref(x, w), what=f"skinny M={M} N={N} K={K}")
+    if N % 8 == 0:
+        wide = torch.zeros(M, N + 8, dtype=BF, device=DEV)
+        hip.linear(x, w, wide[:, :N])
+        assert torch.equal(wide[:, :N], y) and bool((wide[:, N:] == 0).all())
+
+
 @pytest.mark.parametrize("cfg", [144, 212, 222, 242, 244, 412, 422, 442])
 def test_linear_gemv_every_launch_configuration(hip, cfg):
     x = rnd(4, 3584, seed=10)
