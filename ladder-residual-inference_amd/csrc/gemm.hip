@@ -125,112 +125,113 @@ __global__ __launch_bounds__(256) void k_gemm(const u16* __restrict__ x, int64_t
 
 // ---------------------------------------------------------------------------------------------
 // Skinny GEMM for decode batches (4 < M <= 64): the weights are streamed once, the few input rows
-// ride along.  A workgroup owns 32 weight rows (N / 32 workgroups: every CU has work even for the
-// 1280-row wqkv), stages [32 x 128] weight and [MT x 128] input tiles through LDS (coalesced
-// 16-byte loads, double buffered) and its 4 waves split the tile's 8 k-steps; their partial
-// accumulators meet in LDS at the end.  y^T = W x^T on the matrix cores: A = weight rows,
-// B = input rows (MT / 32 column tiles), so a lane ends up with 4 consecutive n of one m.
+// ride along from L2.  y^T = W x^T on the matrix cores: A = 32 weight rows, B = input rows (MT / 32
+// column tiles), so a lane ends up with 4 consecutive n of one m.  A workgroup owns 32 weight rows
+// (N / 32 workgroups: every CU has work even for the 1280-row wqkv) and its 8 waves split K in
+// 64-element chunks (wave w takes chunks w, w + 8, ...: together they read 1 KiB contiguous per
+// row and round).  Both operands are loaded straight into the MFMA register layout (a lane's 8
+// consecutive k of its row: 16 bytes), no LDS staging; each wave keeps PF chunks (PF x 4 KiB of
+// weights) in flight, so a CU has 64+ KiB of weight loads outstanding -- what a latency-bound
+// stream needs.  The waves' partial accumulators meet in LDS at the end, summed in a fixed order.
 // ---------------------------------------------------------------------------------------------
-constexpr int SN = 32, SK = 128, SLD = SK + 8;
+constexpr int SN = 32;       // weight rows per workgroup
+constexpr int SW = 8;        // waves per workgroup
+constexpr int SCH = 64;      // k elements per chunk (4 MFMA k-steps)
+constexpr int SPF = 2;       // chunks in flight per wave beyond the one being multiplied
 
 template <int MT>
-__global__ __launch_bounds__(256) void k_gemm_skinny(const u16* __restrict__ x, int64_t ldx, const u16* __restrict__ w,
-                                                     u16* __restrict__ y, int64_t ldy, int M, int N, int K) {
-  constexpr int CT = MT / 32;                       // column tiles (input rows / 32)
-  constexpr int XCH = MT * SK / 8 / 256;            // 16-byte chunks of the input tile per thread
-  constexpr int WCH = SN * SK / 8 / 256;            // ... of the weight tile
-  constexpr int STAGE = (SN + MT) * SLD;            // elements per LDS stage
-  constexpr int LDS_ELEMS = 2 * STAGE > 4 * CT * 16 * 64 * 2 ? 2 * STAGE : 4 * CT * 16 * 64 * 2;
-  __shared__ __attribute__((aligned(16))) u16 lds[LDS_ELEMS];
+__global__ __launch_bounds__(SW * 64) void k_gemm_skinny(const u16* __restrict__ x, int64_t ldx,
+                                                         const u16* __restrict__ w, u16* __restrict__ y, int64_t ldy,
+                                                         int M, int N, int K) {
+  constexpr int CT = MT / 32;
+  __shared__ __attribute__((aligned(16))) float red[SW * CT * 16 * 64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n0 = blockIdx.x * SN;
-  const int arow = lane & 31, akq = (lane >> 5) * 8;
-
+  const int r = lane & 31, half = lane >> 5;
+  const int n = n0 + r;
+  const bool nok = n < N;
+  const u16* wrow = w + (int64_t)(nok ? n : 0) * K;
+  const u16* xrow[CT];
+  bool mok[CT];
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+    mok[c] = c * 32 + r < M;
+    xrow[c] = x + (int64_t)(mok[c] ? c * 32 + r : 0) * ldx;
+  }
   f32x16_t acc[CT];
 #pragma unroll
   for (int c = 0; c < CT; ++c)
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[c][v] = 0.0f;
 
-  uint4 xr[XCH], wr[WCH];
-  auto fetch = [&](int k0) {
+  struct Chunk {
+    uint4 a[4];
+    uint4 b[CT][4];
+  };
+  auto fetch = [&](int ci, Chunk& ch) {  // chunk index ci of this wave -> elements [k0, k0 + 64)
+    const int k0 = (ci * SW + wave) * SCH;
 #pragma unroll
-    for (int i = 0; i < WCH; ++i) {
-      const int id = tid + i * 256, r = id >> 4, c = (id & 15) * 8;
-      wr[i] = load_w_chunk(w, N, K, n0 + r, k0 + c);
-    }
+    for (int s4 = 0; s4 < 4; ++s4) {
+      const int k = k0 + s4 * 16 + half * 8;
+      const bool kok = k < K;
+      ch.a[s4] = (nok && kok) ? ld16(wrow + k) : make_uint4(0, 0, 0, 0);
 #pragma unroll
-    for (int i = 0; i < XCH; ++i) {
-      const int id = tid + i * 256, r = id >> 4, c = (id & 15) * 8;
-      xr[i] = load_x_chunk<false>(x, ldx, M, K, r, k0 + c);
+      for (int c = 0; c < CT; ++c) ch.b[c][s4] = (mok[c] && kok) ? ld16(xrow[c] + k) : make_uint4(0, 0, 0, 0);
     }
   };
-  auto stage = [&](int buf) {
-    u16* ws_ = lds + buf * STAGE;
-    u16* xs_ = ws_ + SN * SLD;
+  auto mul = [&](const Chunk& ch) {
 #pragma unroll
-    for (int i = 0; i < WCH; ++i) {
-      const int id = tid + i * 256, r = id >> 4, c = (id & 15) * 8;
-      st16(&ws_[r * SLD + c], wr[i]);
-    }
-#pragma unroll
-    for (int i = 0; i < XCH; ++i) {
-      const int id = tid + i * 256, r = id >> 4, c = (id & 15) * 8;
-      st16(&xs_[r * SLD + c], xr[i]);
-    }
-  };
-  const int nk = (K + SK - 1) / SK;
-  fetch(0);
-  stage(0);
-  __syncthreads();
-  for (int kt = 0; kt < nk; ++kt) {
-    const int cur = kt & 1;
-    if (kt + 1 < nk) fetch((kt + 1) * SK);
-    const u16* ws_ = lds + cur * STAGE;
-    const u16* xs_ = ws_ + SN * SLD;
-#pragma unroll
-    for (int q = 0; q < 2; ++q) {  // this wave's two k-steps of the tile
-      const int kk = (wave * 2 + q) * 16;
-      const bf16x8_t af = *reinterpret_cast<const bf16x8_t*>(&ws_[arow * SLD + kk + akq]);
+    for (int s4 = 0; s4 < 4; ++s4) {
+      const u32x4_t av = {ch.a[s4].x, ch.a[s4].y, ch.a[s4].z, ch.a[s4].w};
 #pragma unroll
       for (int c = 0; c < CT; ++c) {
-        const bf16x8_t bfr = *reinterpret_cast<const bf16x8_t*>(&xs_[(c * 32 + arow) * SLD + kk + akq]);
-        acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bfr, acc[c], 0, 0, 0);
+        const u32x4_t bv = {ch.b[c][s4].x, ch.b[c][s4].y, ch.b[c][s4].z, ch.b[c][s4].w};
+        acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, bv),
+                                                        acc[c], 0, 0, 0);
       }
     }
-    if (kt + 1 < nk) stage(cur ^ 1);
-    __syncthreads();
+  };
+  const int nch = (K + SW * SCH - 1) / (SW * SCH);  // chunks per wave (the tail is zero-filled)
+  Chunk c0, c1, c2;
+  fetch(0, c0);
+  fetch(1, c1);
+  int ci = 0;
+  for (; ci + 3 <= nch; ci += 3) {  // three register sets rotate without copies
+    fetch(ci + 2, c2);
+    mul(c0);
+    fetch(ci + 3, c0);
+    mul(c1);
+    fetch(ci + 4, c1);
+    mul(c2);
   }
-  // ---- sum the four waves' partial accumulators in a fixed order
-  float* red = reinterpret_cast<float*>(lds);  // [wave][c][v][lane]
+  if (ci < nch) mul(c0);
+  if (ci + 1 < nch) mul(c1);
+  static_assert(SPF == 2, "the loop above keeps two chunks in flight");
+
+  // ---- sum the waves' partial accumulators in a fixed order
 #pragma unroll
   for (int c = 0; c < CT; ++c)
 #pragma unroll
     for (int v = 0; v < 16; ++v) red[((wave * CT + c) * 16 + v) * 64 + lane] = acc[c][v];
   __syncthreads();
-  // wave w finishes accumulator elements v = 4 w .. 4 w + 3: four consecutive n of one m per lane
+  // wave w finishes accumulator elements v = 2 w, 2 w + 1: two consecutive n of one m per lane
 #pragma unroll
   for (int c = 0; c < CT; ++c) {
-    float o[4];
+    float o[2];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int v = wave * 4 + j;
-      o[j] = (red[((0 * CT + c) * 16 + v) * 64 + lane] + red[((1 * CT + c) * 16 + v) * 64 + lane]) +
-             (red[((2 * CT + c) * 16 + v) * 64 + lane] + red[((3 * CT + c) * 16 + v) * 64 + lane]);
+    for (int j = 0; j < 2; ++j) {
+      const int v = wave * 2 + j;
+      float t = 0.0f;
+#pragma unroll
+      for (int ww = 0; ww < SW; ++ww) t += red[((ww * CT + c) * 16 + v) * 64 + lane];
+      o[j] = t;
     }
     // element v: n = n0 + (v / 4) * 8 + (lane / 32) * 4 + v % 4,  m = c * 32 + lane % 32
-    const int m = c * 32 + (lane & 31), n = n0 + wave * 8 + (lane >> 5) * 4;
+    const int v0 = wave * 2;
+    const int m = c * 32 + r, nn = n0 + (v0 / 4) * 8 + half * 4 + (v0 % 4);
     if (m < M) {
-      if (n + 3 < N) {
-        uint2 pk;
-        pk.x = pack_bf2(o[0], o[1]);
-        pk.y = pack_bf2(o[2], o[3]);
-        *reinterpret_cast<uint2*>(y + (int64_t)m * ldy + n) = pk;
-      } else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          if (n + j < N) y[(int64_t)m * ldy + n + j] = f_to_bf(o[j]);
-      }
+      if (nn + 1 < N) *reinterpret_cast<u32*>(y + (int64_t)m * ldy + nn) = pack_bf2(o[0], o[1]);
+      else if (nn < N) y[(int64_t)m * ldy + nn] = f_to_bf(o[0]);
     }
   }
 }
@@ -245,12 +246,12 @@ extern "C" int lr_linear(const void* x, int64_t ldx, const void* w, void* y, int
   if (K % 8 || ldx % 8) return LR_E_ALIGN;
   hipStream_t s = (hipStream_t)stream;
   if (M <= 4 || (act_swiglu && M <= 8)) return lr_gemv_dispatch(x, ldx, w, y, ldy, M, N, K, act_swiglu, s);
-  if (!act_swiglu && M <= 64 && ldy % 4 == 0) {
+  if (!act_swiglu && M <= 64 && ldy % 2 == 0) {
     const dim3 sgrid((N + SN - 1) / SN);
     if (M <= 32)
-      k_gemm_skinny<32><<<sgrid, dim3(256), 0, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy, M, N, K);
+      k_gemm_skinny<32><<<sgrid, dim3(SW * 64), 0, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy, M, N, K);
     else
-      k_gemm_skinny<64><<<sgrid, dim3(256), 0, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy, M, N, K);
+      k_gemm_skinny<64><<<sgrid, dim3(SW * 64), 0, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy, M, N, K);
     return lr_launch_status();
   }
   const dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
