@@ -222,7 +222,12 @@ def test_prefill_last_logits_only_equals_full():
     full = model(idx, pos)[:, -1].clone()
     model.last_logits_only = True
     last = model(idx, pos)
-    assert last.shape == (2, 1, 512) and torch.equal(last[:, 0], full)
+    assert last.shape == (2, 1, 512)
+    # the two runs push different row counts through the lm_head (34 rows: matrix-core GEMM, 2 rows:
+    # GEMV), i.e. different fp32 summation orders: equal up to one bf16 rounding step in a few places
+    got, want = last[:, 0].float(), full.float()
+    ulp = want.abs().clamp_min(1e-30).log2().floor().exp2() * 2.0 ** -7
+    assert bool(((got - want).abs() <= ulp).all()) and (got == want).float().mean().item() >= 0.9
 
 
 # ---------------------------------------------------------------------------------------------------
