@@ -10,22 +10,45 @@
 
 constexpr int GEMV_WPB = 4;  // waves per workgroup
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+// c + a.lo * b.lo + a.hi * b.hi on packed bf16 pairs, fp32 accumulation (v_dot2_f32_bf16)
+__device__ __forceinline__ float dot2(u32 a, u32 b, float c) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
+}
+
+// 8 inputs of every row as packed bf16 pairs (the SwiGLU values are bf16 by definition)
 template <int M, bool SWIGLU>
 __device__ __forceinline__ void load_x(const u16* __restrict__ x, int64_t ldx, int K, int k, int m_real,
-                                       float (&xf)[M][8]) {
+                                       uint4 (&xp)[M]) {
 #pragma unroll
   for (int m = 0; m < M; ++m) {
     const int mm = m < m_real ? m : m_real - 1;
     if (SWIGLU) {
-      float u[8], g[8];
+      float u[8], g[8], o[8];
       unpack8(ld16(x + mm * ldx + k), u);
       unpack8(ld16(x + mm * ldx + K + k), g);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) xf[m][j] = swiglu_bf(u[j], g[j]);
+      for (int j = 0; j < 8; ++j) o[j] = swiglu_bf(u[j], g[j]);
+      xp[m] = pack8(o);
     } else {
-      unpack8(ld16(x + mm * ldx + k), xf[m]);
+      xp[m] = ld16(x + mm * ldx + k);
     }
   }
+}
+// acc[r][m] += w[r] . x[m] over 8 elements: weights and inputs stay packed, 4 dot2 per pair of rows
+template <int M, int R>
+__device__ __forceinline__ void mac8(const uint4 (&wv)[R], const uint4 (&xp)[M], float (&acc)[R][M]) {
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      float a = acc[r][m];
+      a = dot2(wv[r].x, xp[m].x, a);
+      a = dot2(wv[r].y, xp[m].y, a);
+      a = dot2(wv[r].z, xp[m].z, a);
+      a = dot2(wv[r].w, xp[m].w, a);
+      acc[r][m] = a;
+    }
 }
 
 template <int M, int R, int KSPLIT, int U, bool SWIGLU>
@@ -62,17 +85,9 @@ __global__ __launch_bounds__(GEMV_WPB * 64) void k_gemv(const u16* __restrict__ 
       for (int r = 0; r < R; ++r) wv[u][r] = ld16(wrow[r] + k + u * KSTEP);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      float xf[M][8];
-      load_x<M, SWIGLU>(x, ldx, K, k + u * KSTEP, m_real, xf);
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        float wf[8];
-        unpack8(wv[u][r], wf);
-#pragma unroll
-        for (int m = 0; m < M; ++m)
-#pragma unroll
-          for (int j = 0; j < 8; ++j) acc[r][m] = fmaf(wf[j], xf[m][j], acc[r][m]);
-      }
+      uint4 xp[M];
+      load_x<M, SWIGLU>(x, ldx, K, k + u * KSTEP, m_real, xp);
+      mac8<M, R>(wv[u], xp, acc);
     }
   }
   // remainder steps
@@ -80,17 +95,9 @@ __global__ __launch_bounds__(GEMV_WPB * 64) void k_gemv(const u16* __restrict__ 
     uint4 wv[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) wv[r] = ld16(wrow[r] + k);
-    float xf[M][8];
-    load_x<M, SWIGLU>(x, ldx, K, k, m_real, xf);
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      float wf[8];
-      unpack8(wv[r], wf);
-#pragma unroll
-      for (int m = 0; m < M; ++m)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) acc[r][m] = fmaf(wf[j], xf[m][j], acc[r][m]);
-    }
+    uint4 xp[M];
+    load_x<M, SWIGLU>(x, ldx, K, k, m_real, xp);
+    mac8<M, R>(wv, xp, acc);
   }
 
 #pragma unroll
