@@ -76,6 +76,9 @@ def main():
     ap.add_argument("--prompt", type=int, default=2048)
     ap.add_argument("--model", type=str, default="gpt_ladder:ladder-70b-tp8")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--per-op", action="store_true",
+                    help="decode with one kernel per operation (captured in the hipGraph) instead of the persistent "
+                         "one-kernel step: the comparison point, not the headline")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (reads 1 GiB, writes 1 GiB) a few times: under "
                          "rocprofv3 --pmc its FETCH_SIZE / WRITE_SIZE readings calibrate the counters' unit")
@@ -96,6 +99,8 @@ def main():
     B, T, K, W = args.batch, args.prompt, args.steps, args.warmup
     model = bm._load_model(args.model, dev, torch.bfloat16, seed=0, verbose=False)
     model.last_logits_only = True          # prefill is set-up here, not the timed region
+    if args.per_op:
+        model.use_fused_step = False
     cfg = model.config
     new = max(K, W, 127) + 1
     g = torch.Generator(device=dev)
@@ -186,7 +191,8 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{args.model} rank shard (dim {cfg.dim}, {cfg.n_layer} layers, {cfg.n_head_local} q / "
                                f"{cfg.n_kv_local} kv heads, FFN {cfg.ffn_local}, lm_head rows {cfg.output_rows}), "
-                               f"batch {B}, prompt {T}, greedy decode, hipGraph replay per step",
+                               f"batch {B}, prompt {T}, greedy decode, hipGraph replay per step"
+                               + (", one kernel per operation" if args.per_op else ""),
                    "batch": B, "prompt_len": T, "virtual_tp": cfg.tp_world_size},
         "ms_per_token": round(ms_per_step, 4),
         "prefill_s": round(prefill_s, 4),

@@ -400,7 +400,7 @@ FORWARD = {"ladder": forward_ladder, "dense": forward_dense, "desync": forward_d
 
 def greedy(logits: Tensor) -> Tensor:
     """argmax of the last position, first maximum on ties -> int32 [B, 1].  Stands where
-    benchmark.py:73-77 samples (BASELINE asks for greedy decoding)."""
+    benchmark.py:73-77 samples; the parity contract of this build is greedy decoding."""
     return torch.argmax(logits[:, -1], dim=-1, keepdim=True).to(torch.int32)
 
 
