@@ -168,6 +168,15 @@ int lr_ladder_decode_step(const lr_ladder_model_t* model, int batch, const int32
                           int64_t ld_hist, int hist_len, int pos0, void* workspace, size_t bytes, lr_stream_t stream);
 size_t lr_ladder_step_fail_offset(void);
 
+/* benchmark.py:58-77 (sample, logits_to_probs, multinomial_sample_one_no_sync) on the bf16 logits of
+ * the last position, one row per sequence: s = bf16(logits * (1 / max(temperature, 1e-5))); values
+ * below the top_k-th largest become -inf (top_k <= 0: no cut; top_k > V: V); probs = bf16 softmax
+ * of s (fp32 inside); next_token[b] = argmax_i bf16(probs[i] / noise[i]) (lowest index among equals).
+ * `noise` holds the caller's Exp(1) draws (bf16 [B][ldn]; the reference draws them with
+ * torch.empty_like(probs).exponential_(1), benchmark.py:59), `probs` is optional (bf16 [B][ldp]). */
+int lr_sample_topk(const void* logits, int64_t ldl, const void* noise, int64_t ldn, int B, int V, float temperature,
+                   int top_k, void* probs, int64_t ldp, int32_t* next_token, lr_stream_t stream);
+
 /* Tuning hook, no counterpart in the reference: use at least this many attention workgroups in
  * the step kernel (more workgroups, fewer keys each; <= 0 restores the default).  Set it before the
  * workspace is sized and initialised. */

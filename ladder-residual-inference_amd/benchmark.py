@@ -74,7 +74,9 @@ def sample(logits, temperature: float = 1.0, top_k: Optional[int] = None, greedy
         if model is not None:
             return model.greedy_next(logits), None            # lr_argmax on the device
         return torch.argmax(logits[:, -1], dim=-1, keepdim=True).to(torch.int), None
-    probs = logits_to_probs(logits[:, -1].float(), temperature, top_k)
+    if model is not None and logits.is_cuda and logits.dtype == torch.bfloat16:
+        return model.sample_next(logits, temperature, top_k)  # lr_sample_topk on the device
+    probs = logits_to_probs(logits[:, -1], temperature, top_k)
     return multinomial_sample_one_no_sync(probs), probs
 
 

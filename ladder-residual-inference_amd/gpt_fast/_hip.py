@@ -30,6 +30,8 @@ _PROTOS = {
     "lr_attn_prefill": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,
                                 c_int, c_int, c_int, c_int, c_void_p]),
     "lr_argmax": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_int, c_void_p]),
+    "lr_sample_topk": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_float, c_int, c_void_p, c_int64,
+                               c_void_p, c_void_p]),
     "lr_advance": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "lr_gemv_set_cfg": (None, [c_int]),
     "lr_ladder_step_workspace_bytes": (c_size_t, [c_void_p, c_int]),
@@ -209,6 +211,22 @@ def argmax(logits: torch.Tensor, out: torch.Tensor):
     B, V, ld = _rows_ld(logits)
     assert out.dtype == torch.int32 and out.numel() == B and out.is_cuda
     _check(load().lr_argmax(_dev(logits), ld, out.data_ptr(), B, V, _stream()), "lr_argmax")
+    return out
+
+
+def sample_topk(logits: torch.Tensor, noise: torch.Tensor, temperature: float, top_k, out: torch.Tensor,
+                probs: torch.Tensor = None):
+    """Temperature / top-k / softmax / exponential-race draw of benchmark.py:58-77 on bf16 rows [B, V];
+    `noise` are the caller's Exp(1) draws (bf16 [B, V]); writes int32 tokens to `out` (and bf16 `probs`)."""
+    B, V, ld = _rows_ld(logits)
+    assert noise.dtype == torch.bfloat16 and noise.is_cuda and noise.shape == (B, V) and noise.stride(1) == 1
+    assert out.dtype == torch.int32 and out.numel() == B and out.is_cuda
+    if probs is not None:
+        assert probs.dtype == torch.bfloat16 and probs.is_cuda and probs.shape == (B, V) and probs.stride(1) == 1
+    _check(load().lr_sample_topk(_dev(logits), ld, noise.data_ptr(), noise.stride(0), B, V, float(temperature),
+                                 int(top_k) if top_k is not None else 0,
+                                 None if probs is None else probs.data_ptr(), 0 if probs is None else probs.stride(0),
+                                 out.data_ptr(), _stream()), "lr_sample_topk")
     return out
 
 

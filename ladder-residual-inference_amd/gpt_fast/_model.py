@@ -172,3 +172,13 @@ class GPTBase(nn.Module):
         out = ws.next_token if ws.next_token.shape[0] == B else torch.empty(B, 1, dtype=torch.int32,
                                                                             device=logits.device)
         return _hip.argmax(logits[:, -1], out)
+
+    def sample_next(self, logits: Tensor, temperature: float, top_k) -> tuple:
+        """benchmark.py:58-77 on the last position of bf16 `logits` [B, S, V] -> (int32 [B, 1], probs [B, V]).
+        The Exp(1) noise comes from torch's generator exactly as in the reference (same shape and dtype)."""
+        last = logits[:, -1]
+        probs = torch.empty(last.shape, dtype=last.dtype, device=last.device)
+        noise = torch.empty_like(probs).exponential_(1)
+        out = torch.empty(last.shape[0], 1, dtype=torch.int32, device=last.device)
+        _hip.sample_topk(last, noise, temperature, top_k, out, probs)
+        return out, probs

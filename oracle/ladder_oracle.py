@@ -404,6 +404,23 @@ def greedy(logits: Tensor) -> Tensor:
     return torch.argmax(logits[:, -1], dim=-1, keepdim=True).to(torch.int32)
 
 
+def sample_topk(last_logits: Tensor, noise: Tensor, temperature: float = 1.0, top_k: Optional[int] = None):
+    """benchmark.py:58-77 (sample / logits_to_probs / multinomial_sample_one_no_sync) on the logits of
+    the last position [B, V], with the Exp(1) draws of :59 passed in as `noise` [B, V] so that a run can
+    be repeated:  scale by 1 / max(T, 1e-5) (:64), everything below the top_k-th largest value to -inf
+    (:66-69, ties with the pivot stay), softmax (:70), token = argmax(probs / noise) (:60).
+    Works in the dtype of `last_logits` (the reference samples from bf16 logits), on its device.
+    Returns (int32 [B, 1], probs [B, V])."""
+    s = last_logits / max(temperature, 1e-5)
+    if top_k is not None:
+        k = min(int(top_k), s.size(-1))
+        pivot = torch.topk(s, k, dim=-1).values[..., k - 1:k]
+        s = s.masked_fill(s < pivot, float("-inf"))
+    probs = torch.softmax(s, dim=-1)
+    token = torch.argmax(probs / noise, dim=-1, keepdim=True).to(torch.int32)
+    return token, probs
+
+
 @torch.no_grad()
 def generate(cfg: OracleConfig, P: Dict[str, Tensor], prompt: Tensor, max_new_tokens: int, batch_size: int,
              family: str = "ladder", caches: Optional[OracleCaches] = None, forced: Optional[Tensor] = None,
