@@ -124,6 +124,166 @@ __global__ __launch_bounds__(256) void k_gemm(const u16* __restrict__ x, int64_t
 }
 
 // ---------------------------------------------------------------------------------------------
+// Large-tile variant for prefill-sized problems (M >= 512): workgroup tile 256 x 256 x 64, four
+// waves in a 2 x 2 arrangement, each owning 128 x 128 = 4 x 4 MFMA tiles (256 accumulator
+// registers; one workgroup per CU, so a wave has the whole 512-register budget).  The point is LDS
+// traffic: a 64 x 64 wave tile reads 1 KiB of LDS per MFMA, which at 128 B/clk per CU takes as long
+// as the MFMAs themselves; a 128 x 128 wave tile reads half of that.  Staging is the same as in
+// k_gemm (128-bit global loads -> registers -> padded LDS rows, double-buffered, next tile's
+// loads in flight during the multiply).  Tiles are dealt so that the 32 workgroups an XCD runs
+// together cover 4 row tiles x 8 column tiles: they share operand rows in that XCD's L2
+// (blockIdx % 8 is the XCD), which keeps the HBM demand ~5x below the L2 demand.
+// ---------------------------------------------------------------------------------------------
+constexpr int GM = 256, GN = 256;
+
+__global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int64_t ldx, const u16* __restrict__ w,
+                                                  u16* __restrict__ y, int64_t ldy, int M, int N, int K, int tm,
+                                                  int tn) {
+  extern __shared__ __attribute__((aligned(16))) u16 gsm[];
+  u16* xs = gsm;                      // [2][GM * LDT]
+  u16* ws = gsm + 2 * GM * LDT;       // [2][GN * LDT]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  // ---- tile of this workgroup
+  int mt, nt;
+  {
+    const int id = blockIdx.x;
+    if (tm % 32 == 0) {  // XCD-aware: XCD x owns a band of tm / 8 row tiles, walked 4 row tiles x all column tiles at a time
+      const int xcd = id & 7, j = id >> 3;
+      const int per_group = 4 * tn;
+      const int grp = j / per_group, r = j - grp * per_group;
+      mt = xcd * (tm / 8) + grp * 4 + (r & 3);
+      nt = r >> 2;
+    } else {
+      mt = id / tn;
+      nt = id - mt * tn;
+    }
+  }
+  const int m0 = mt * GM, n0 = nt * GN;
+
+  // staging assignment: 2048 16-byte chunks per operand tile, 8 per thread
+  f32x16_t acc[4][4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
+
+  const int srow0 = tid >> 3, scol = (tid & 7) * 8;  // chunk i sits 32 rows below chunk i - 1
+  // Operand rows are read through buffer resources based at the tile's first row; a chunk beyond M,
+  // N or K gets an offset outside the resource and reads as zero: no branches around the loads.
+  const __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc(const_cast<u16*>(x + (int64_t)m0 * ldx), 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc(const_cast<u16*>(w + (int64_t)n0 * K), 0, 0x7fffffff, 0x00020000);
+  int xoff[8], woff[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int r = srow0 + i * 32;
+    xoff[i] = m0 + r < M ? (int)((int64_t)r * ldx * 2) : (int)0x80000000;
+    woff[i] = n0 + r < N ? r * K * 2 : (int)0x80000000;
+  }
+  auto fetch = [&](const __amdgpu_buffer_rsrc_t& res, int rowoff, int k) -> uint4 {
+    const int off = (k < K && rowoff >= 0) ? rowoff + k * 2 : (int)0x80000000;
+    const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(res, off, 0, 0);
+    return make_uint4(v.x, v.y, v.z, v.w);
+  };
+  uint4 xr[8], wr[8];
+  const int nk = (K + BK - 1) / BK;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    xr[i] = fetch(xres, xoff[i], scol);
+    wr[i] = fetch(wres, woff[i], scol);
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    st16(&xs[(srow0 + i * 32) * LDT + scol], xr[i]);
+    st16(&ws[(srow0 + i * 32) * LDT + scol], wr[i]);
+  }
+  __syncthreads();
+
+  const int arow = lane & 31, akq = (lane >> 5) * 8;
+  for (int kt = 0; kt < nk; ++kt) {
+    const int cur = kt & 1;
+    const u16* xc = xs + cur * GM * LDT;
+    const u16* wc = ws + cur * GN * LDT;
+    if (kt + 1 < nk) {
+      const int k0 = (kt + 1) * BK;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        xr[i] = fetch(xres, xoff[i], k0 + scol);
+        wr[i] = fetch(wres, woff[i], k0 + scol);
+      }
+    }
+    // the fragments of k-step kk + 1 are read from LDS while the 16 MFMAs of k-step kk run
+    bf16x8_t af[2][4], bfr[2][4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+      af[0][a] = *reinterpret_cast<const bf16x8_t*>(&xc[(wm * 128 + a * 32 + arow) * LDT + akq]);
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+      bfr[0][b] = *reinterpret_cast<const bf16x8_t*>(&wc[(wn * 128 + b * 32 + arow) * LDT + akq]);
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      const int c = ks & 1, nx = c ^ 1;
+      __builtin_amdgcn_sched_barrier(0);
+      if (ks + 1 < BK / 16) {
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+          af[nx][a] = *reinterpret_cast<const bf16x8_t*>(&xc[(wm * 128 + a * 32 + arow) * LDT + (ks + 1) * 16 + akq]);
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+          bfr[nx][b] = *reinterpret_cast<const bf16x8_t*>(&wc[(wn * 128 + b * 32 + arow) * LDT + (ks + 1) * 16 + akq]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[c][a], bfr[c][b], acc[a][b], 0, 0, 0);
+    }
+    if (kt + 1 < nk) {
+      u16* xn = xs + (cur ^ 1) * GM * LDT;
+      u16* wn_ = ws + (cur ^ 1) * GN * LDT;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        st16(&xn[(srow0 + i * 32) * LDT + scol], xr[i]);
+        st16(&wn_[(srow0 + i * 32) * LDT + scol], wr[i]);
+      }
+    }
+    __syncthreads();
+  }
+
+  // accumulator element v of a 32x32 tile: row = (v / 4) * 8 + (lane / 32) * 4 + v % 4, col = lane % 32
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int n = n0 + wn * 128 + b * 32 + (lane & 31);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + wm * 128 + a * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+        if (m < M && n < N) y[(int64_t)m * ldy + n] = f_to_bf(acc[a][b][v]);
+      }
+    }
+}
+
+static int launch_gemm_big(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
+                           hipStream_t s) {
+  constexpr size_t lds = (size_t)2 * (GM + GN) * LDT * sizeof(u16);
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_big), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess)
+      return LR_E_LAUNCH;
+    attr_set = true;
+  }
+  const int tm = (M + GM - 1) / GM, tn = (N + GN - 1) / GN;
+  k_gemm_big<<<dim3((unsigned)(tm * tn)), dim3(256), lds, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy, M, N, K,
+                                                              tm, tn);
+  return lr_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
 // Skinny GEMM for decode batches (4 < M <= 64): the weights are streamed once, the few input rows
 // ride along from L2.  y^T = W x^T on the matrix cores: A = 32 weight rows, B = input rows (MT / 32
 // column tiles), so a lane ends up with 4 consecutive n of one m.  A workgroup owns 32 weight rows
@@ -254,6 +414,9 @@ extern "C" int lr_linear(const void* x, int64_t ldx, const void* w, void* y, int
       k_gemm_skinny<64><<<sgrid, dim3(SW * 64), 0, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy, M, N, K);
     return lr_launch_status();
   }
+  if (!act_swiglu && M >= 512 && N >= 256 && ((M + GM - 1) / GM) * ((N + GN - 1) / GN) >= 192 &&
+      (int64_t)GM * ldx * 2 < 0x7fffffff && (int64_t)GN * K * 2 < 0x7fffffff)
+    return launch_gemm_big(x, ldx, w, y, ldy, M, N, K, s);
   const dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
   if (grid.y > 65535) return LR_E_UNSUPPORTED;
   if (act_swiglu)

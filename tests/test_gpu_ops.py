@@ -190,7 +190,11 @@ def test_linear_gemv_is_deterministic(hip):
 
 
 @pytest.mark.parametrize("M,N,K", [(9, 256, 64), (128, 128, 64), (130, 1280, 8192), (2048, 1280, 1024),
-                                   (333, 1001, 520), (64, 16032, 2048), (16, 8192, 3584), (257, 384, 8)])
+                                   (333, 1001, 520), (64, 16032, 2048), (16, 8192, 3584), (257, 384, 8),
+                                   # 256 x 256 tiles (M >= 512): whole tiles, ragged edges in M, N and K, the
+                                   # XCD-aware tile order (M / 256 a multiple of 32) and the plain one
+                                   (512, 256, 64), (700, 500, 328), (1024, 6144, 4096), (8192, 512, 136),
+                                   (8192 + 3, 257, 72)])
 def test_linear_gemm(hip, M, N, K):
     x = rnd(M, K, seed=14)
     w = rnd(N, K, seed=15, scale=0.02)
