@@ -8,6 +8,7 @@
 // reads that deliver exactly the 8 consecutive k an MFMA lane feeds.  LDS is double-buffered and
 // the global loads of tile t+1 are in flight while tile t is multiplied.
 #include "lr_common.h"
+#include <type_traits>
 
 int lr_gemv_dispatch(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
                      int act_swiglu, hipStream_t s);
@@ -187,6 +188,10 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
     const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(res, off, 0, 0);
     return make_uint4(v.x, v.y, v.z, v.w);
   };
+  // Global -> LDS staging one tile ahead through ONE register set, in quarters: while tile kt is
+  // multiplied, quarter q of tile kt + 1 (requested a whole iteration earlier, so it has landed) is
+  // written to the other LDS buffer behind the MFMA group of k-step q, and the same registers are
+  // at once refilled with quarter q of tile kt + 2.
   uint4 xr[8], wr[8];
   const int nk = (K + BK - 1) / BK;
 #pragma unroll
@@ -199,6 +204,13 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
     st16(&xs[(srow0 + i * 32) * LDT + scol], xr[i]);
     st16(&ws[(srow0 + i * 32) * LDT + scol], wr[i]);
   }
+  // (requests beyond K read as zero: every load and LDS write below is unconditional, so the number of
+  // loads in flight never depends on a branch and the waits can be exact)
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    xr[i] = fetch(xres, xoff[i], BK + scol);
+    wr[i] = fetch(wres, woff[i], BK + scol);
+  }
   __syncthreads();
 
   const int arow = lane & 31, akq = (lane >> 5) * 8;
@@ -206,15 +218,10 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
     const int cur = kt & 1;
     const u16* xc = xs + cur * GM * LDT;
     const u16* wc = ws + cur * GN * LDT;
-    if (kt + 1 < nk) {
-      const int k0 = (kt + 1) * BK;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        xr[i] = fetch(xres, xoff[i], k0 + scol);
-        wr[i] = fetch(wres, woff[i], k0 + scol);
-      }
-    }
-    // the fragments of k-step kk + 1 are read from LDS while the 16 MFMAs of k-step kk run
+    u16* xn = xs + (cur ^ 1) * GM * LDT;
+    u16* wn_ = ws + (cur ^ 1) * GN * LDT;
+    const int k2 = (kt + 2) * BK;
+    // the fragments of k-step ks + 1 are read from LDS while the 16 MFMAs of k-step ks run
     bf16x8_t af[2][4], bfr[2][4];
 #pragma unroll
     for (int a = 0; a < 4; ++a)
@@ -240,14 +247,16 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
 #pragma unroll
         for (int b = 0; b < 4; ++b)
           acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[c][a], bfr[c][b], acc[a][b], 0, 0, 0);
-    }
-    if (kt + 1 < nk) {
-      u16* xn = xs + (cur ^ 1) * GM * LDT;
-      u16* wn_ = ws + (cur ^ 1) * GN * LDT;
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 2 * ks; i < 2 * ks + 2; ++i) {
         st16(&xn[(srow0 + i * 32) * LDT + scol], xr[i]);
         st16(&wn_[(srow0 + i * 32) * LDT + scol], wr[i]);
+      }
+#pragma unroll
+      for (int i = 2 * ks; i < 2 * ks + 2; ++i) {
+        xr[i] = fetch(xres, xoff[i], k2 + scol);
+        wr[i] = fetch(wres, woff[i], k2 + scol);
       }
     }
     __syncthreads();
