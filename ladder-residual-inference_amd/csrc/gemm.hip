@@ -246,7 +246,7 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
       for (int a = 0; a < 4; ++a)
 #pragma unroll
         for (int b = 0; b < 4; ++b)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[c][a], bfr[c][b], acc[a][b], 0, 0, 0);
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[c][b], af[c][a], acc[a][b], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 2 * ks; i < 2 * ks + 2; ++i) {
@@ -262,18 +262,33 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
     __syncthreads();
   }
 
-  // accumulator element v of a 32x32 tile: row = (v / 4) * 8 + (lane / 32) * 4 + v % 4, col = lane % 32
+  // The products were formed as W-tile x X-tile^T, so accumulator element v of a 32 x 32 tile is
+  // output column n = (v / 4) * 8 + (lane / 32) * 4 + v % 4 of output row m = lane % 32: a lane holds
+  // four consecutive n of one row per group of four registers -> one 8-byte store.
+  const bool vec_ok = (ldy & 3) == 0;
 #pragma unroll
-  for (int a = 0; a < 4; ++a)
+  for (int a = 0; a < 4; ++a) {
+    const int m = m0 + wm * 128 + a * 32 + (lane & 31);
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
-      const int n = n0 + wn * 128 + b * 32 + (lane & 31);
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int m = m0 + wm * 128 + a * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
-        if (m < M && n < N) y[(int64_t)m * ldy + n] = f_to_bf(acc[a][b][v]);
+      for (int g = 0; g < 4; ++g) {
+        const int n = n0 + wn * 128 + b * 32 + g * 8 + (lane >> 5) * 4;
+        if (m < M) {
+          if (vec_ok && n + 3 < N) {
+            uint2 pk;
+            pk.x = pack_bf2(acc[a][b][4 * g], acc[a][b][4 * g + 1]);
+            pk.y = pack_bf2(acc[a][b][4 * g + 2], acc[a][b][4 * g + 3]);
+            *reinterpret_cast<uint2*>(y + (int64_t)m * ldy + n) = pk;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n + e < N) y[(int64_t)m * ldy + n + e] = f_to_bf(acc[a][b][4 * g + e]);
+          }
+        }
       }
     }
+  }
 }
 
 static int launch_gemm_big(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
