@@ -170,13 +170,16 @@ __global__ __launch_bounds__(HD) void k_attn_decode_combine(const float* __restr
   const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
   const float* ml = ml_part + ((int64_t)b * Hq + h) * nsplit * 2;
   const float* op = o_part + ((int64_t)b * Hq + h) * nsplit * HD;
+  // branch-free loops, unrolled: the loads of eight splits are in flight together instead of one
+  // dependent round trip per split
   float M = -INFINITY;
+#pragma unroll 8
   for (int s = 0; s < nsplit; ++s) M = fmaxf(M, ml[2 * s]);
   float L = 0.0f, o = 0.0f;
+#pragma unroll 8
   for (int s = 0; s < nsplit; ++s) {
     const float m = ml[2 * s];
-    if (m == -INFINITY) continue;
-    const float wgt = expf(m - M);
+    const float wgt = m == -INFINITY ? 0.0f : expf(m - M);  // an empty split carries (-inf, 0, 0)
     L = fmaf(wgt, ml[2 * s + 1], L);
     o = fmaf(wgt, op[(int64_t)s * HD + d], o);
   }

@@ -71,25 +71,40 @@ __global__ __launch_bounds__(256) void k_add_rmsnorm(const u16* __restrict__ rin
   __shared__ float red[4];
   const int tid = threadIdx.x;
   const int64_t base = (int64_t)blockIdx.x * dim;
+  // Every load of the row (residual, both addends, gain) is requested before the first one is
+  // used: columns past `dim` are clamped to column 0 and ignored, so no branch separates the loads
+  // and the kernel costs one memory round trip instead of one per iteration.
+  uint4 qr[NORM_MAXIT], q1[NORM_MAXIT], q2[NORM_MAXIT], qg[NORM_MAXIT];
+#pragma unroll
+  for (int it = 0; it < NORM_MAXIT; ++it) {
+    const int c0 = (tid + it * 256) * 8;
+    if (it * 256 * 8 >= dim) break;  // uniform
+    const int c = c0 < dim ? c0 : 0;
+    qr[it] = ld16(rin + base + c);
+    q1[it] = d1 ? ld16(d1 + base + c) : make_uint4(0, 0, 0, 0);
+    q2[it] = d2 ? ld16(d2 + base + c) : make_uint4(0, 0, 0, 0);
+    qg[it] = ld16(gain + c);
+  }
   float r[NORM_MAXIT][8];
   float ss = 0.0f;
 #pragma unroll
   for (int it = 0; it < NORM_MAXIT; ++it) {
     const int c = (tid + it * 256) * 8;
+    if (it * 256 * 8 >= dim) break;
+    unpack8(qr[it], r[it]);
+    if (d1) {
+      float t[8];
+      unpack8(q1[it], t);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) r[it][j] = round_bf(r[it][j] + t[j]);
+    }
+    if (d2) {
+      float t[8];
+      unpack8(q2[it], t);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) r[it][j] = round_bf(r[it][j] + t[j]);
+    }
     if (c < dim) {
-      unpack8(ld16(rin + base + c), r[it]);
-      if (d1) {
-        float t[8];
-        unpack8(ld16(d1 + base + c), t);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) r[it][j] = round_bf(r[it][j] + t[j]);
-      }
-      if (d2) {
-        float t[8];
-        unpack8(ld16(d2 + base + c), t);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) r[it][j] = round_bf(r[it][j] + t[j]);
-      }
       if (rout) st16(rout + base + c, pack8(r[it]));
 #pragma unroll
       for (int j = 0; j < 8; ++j) ss += r[it][j] * r[it][j];
@@ -103,9 +118,10 @@ __global__ __launch_bounds__(256) void k_add_rmsnorm(const u16* __restrict__ rin
 #pragma unroll
   for (int it = 0; it < NORM_MAXIT; ++it) {
     const int c = (tid + it * 256) * 8;
+    if (it * 256 * 8 >= dim) break;
     if (c < dim) {
       float g[8], o[8];
-      unpack8(ld16(gain + c), g);
+      unpack8(qg[it], g);
 #pragma unroll
       for (int j = 0; j < 8; ++j) o[j] = round_bf(r[it][j] * inv) * g[j];
       st16(nout + base + c, pack8(o));
