@@ -352,15 +352,30 @@ __global__ __launch_bounds__(SW * 64) void k_gemm_skinny(const u16* __restrict__
     uint4 a[4];
     uint4 b[CT][4];
   };
+  // buffer resources: weights based at this workgroup's first row, inputs at row 0
+  const __amdgpu_buffer_rsrc_t wres =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<u16*>(w + (int64_t)n0 * K), 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc(const_cast<u16*>(x), 0, 0x7fffffff, 0x00020000);
+  const int woff = r * K * 2;
+  int xoff[CT];
+#pragma unroll
+  for (int c = 0; c < CT; ++c) xoff[c] = (int)((c * 32 + r) * ldx * 2);
   auto fetch = [&](int ci, Chunk& ch) {  // chunk index ci of this wave -> elements [k0, k0 + 64)
     const int k0 = (ci * SW + wave) * SCH;
 #pragma unroll
     for (int s4 = 0; s4 < 4; ++s4) {
       const int k = k0 + s4 * 16 + half * 8;
+      // no branch around a load: what lies beyond N, M or K gets an offset outside the buffer and reads
+      // as zero, so the number of loads in flight is fixed and the waits between chunks are exact
       const bool kok = k < K;
-      ch.a[s4] = (nok && kok) ? ld16(wrow + k) : make_uint4(0, 0, 0, 0);
+      const u32x4_t av = __builtin_amdgcn_raw_buffer_load_b128(wres, (kok && nok) ? woff + k * 2 : (int)0x80000000, 0, 0);
+      ch.a[s4] = make_uint4(av.x, av.y, av.z, av.w);
 #pragma unroll
-      for (int c = 0; c < CT; ++c) ch.b[c][s4] = (mok[c] && kok) ? ld16(xrow[c] + k) : make_uint4(0, 0, 0, 0);
+      for (int c = 0; c < CT; ++c) {
+        const u32x4_t bv =
+            __builtin_amdgcn_raw_buffer_load_b128(xres, (kok && mok[c]) ? xoff[c] + k * 2 : (int)0x80000000, 0, 0);
+        ch.b[c][s4] = make_uint4(bv.x, bv.y, bv.z, bv.w);
+      }
     }
   };
   auto mul = [&](const Chunk& ch) {
@@ -430,7 +445,15 @@ extern "C" int lr_linear(const void* x, int64_t ldx, const void* w, void* y, int
   if (K % 8 || ldx % 8) return LR_E_ALIGN;
   hipStream_t s = (hipStream_t)stream;
   if (M <= 4 || (act_swiglu && M <= 8)) return lr_gemv_dispatch(x, ldx, w, y, ldy, M, N, K, act_swiglu, s);
-  if (!act_swiglu && M <= 64 && ldy % 2 == 0) {
+  if (!act_swiglu && M <= 8 && (N + SN - 1) / SN < 96) {
+    // few weight rows (the wqkv of a rank shard): 32-row workgroups would leave most CUs idle, so the
+    // GEMV kernel (a row per wave, every CU busy) runs twice, four input rows each; the second pass
+    // finds the weights in the memory-side cache
+    const int rc = lr_gemv_dispatch(x, ldx, w, y, ldy, 4, N, K, 0, s);
+    if (rc != LR_OK) return rc;
+    return lr_gemv_dispatch((const u16*)x + 4 * ldx, ldx, w, (u16*)y + 4 * ldy, ldy, M - 4, N, K, 0, s);
+  }
+  if (!act_swiglu && M <= 64 && ldy % 2 == 0 && (int64_t)64 * ldx * 2 < 0x7fffffff && (int64_t)SN * K * 2 < 0x7fffffff) {
     const dim3 sgrid((N + SN - 1) / SN);
     if (M <= 32)
       k_gemm_skinny<32><<<sgrid, dim3(SW * 64), 0, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy, M, N, K);
