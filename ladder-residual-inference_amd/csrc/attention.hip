@@ -411,25 +411,40 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const u16* __restrict
   const u16* kbase = kc + ((int64_t)b * Hkv + kvh) * Smax * HD;
   const u16* vbase = vc + ((int64_t)b * Hkv + kvh) * Smax * HD;
 
+  // Staging: a thread owns one 8-element slice of TWO neighbouring keys (key pair kp, slice dch), so
+  // that V^T can be written as whole dwords (two keys of one dimension).  The pair index is XOR-ed
+  // with 4 * (dch / 4): slices 32 dimensions apart would otherwise fall on the same LDS banks (row
+  // stride 18 dwords, 8 rows per slice).  The next tile's loads are in flight during the products.
+  const int dch = tid % (HD / 8), kp = tid / (HD / 8);
+  const bool stager = kp < 16;
+  const int kps = kp ^ ((dch >> 2) * 4);
+  uint4 gk[2], gv[2];
+  auto stage_load = [&](int t0) {
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int key = t0 + 2 * kp + e;
+      const bool ok = stager && key < nkeys;
+      gk[e] = ok ? ld16(kbase + (int64_t)key * HD + dch * 8) : make_uint4(0, 0, 0, 0);
+      gv[e] = ok ? ld16(vbase + (int64_t)key * HD + dch * 8) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  stage_load(0);
+  u32* vt32 = reinterpret_cast<u32*>(vt);
   for (int t0 = 0; t0 < nkeys; t0 += 32) {
     __syncthreads();
-    // ---- stage 32 keys: K row-major, V transposed ([d][key])
-    for (int c = tid; c < 32 * HD / 8; c += 256) {
-      const int key = c / (HD / 8), d = (c % (HD / 8)) * 8;
-      uint4 kk = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
-      if (t0 + key < nkeys) {
-        kk = ld16(kbase + (int64_t)(t0 + key) * HD + d);
-        vv = ld16(vbase + (int64_t)(t0 + key) * HD + d);
-      }
-      *reinterpret_cast<uint4*>(&ks[key * KROW + d]) = kk;
-      const u32 w4[4] = {vv.x, vv.y, vv.z, vv.w};
+    // ---- 32 keys into LDS: K row-major, V transposed ([d][key], two keys per dword)
+    if (stager) {
+#pragma unroll
+      for (int e = 0; e < 2; ++e) *reinterpret_cast<uint4*>(&ks[(2 * kp + e) * KROW + dch * 8]) = gk[e];
+      const u32 a4[4] = {gv[0].x, gv[0].y, gv[0].z, gv[0].w}, b4[4] = {gv[1].x, gv[1].y, gv[1].z, gv[1].w};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        vt[(d + 2 * j) * VROW + key] = (u16)(w4[j] & 0xffffu);
-        vt[(d + 2 * j + 1) * VROW + key] = (u16)(w4[j] >> 16);
+        vt32[(dch * 8 + 2 * j) * (VROW / 2) + kps] = (a4[j] & 0xffffu) | (b4[j] << 16);
+        vt32[(dch * 8 + 2 * j + 1) * (VROW / 2) + kps] = (a4[j] >> 16) | (b4[j] & 0xffff0000u);
       }
     }
     __syncthreads();
+    stage_load(t0 + 32);
     // ---- S^T tile: rows = keys, columns = queries
     f32x16_t sacc;
 #pragma unroll
@@ -486,8 +501,10 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const u16* __restrict
       for (int v = 0; v < 16; ++v) o[d][v] *= corr;
 #pragma unroll
       for (int h2 = 0; h2 < 2; ++h2) {
-        const u16* vr = &vt[(d * 32 + col) * VROW + 16 * h2 + 4 * half];
-        const uint2 v0 = *reinterpret_cast<const uint2*>(vr), v1 = *reinterpret_cast<const uint2*>(vr + 8);
+        // keys 16 h2 + 4 half + {0..3} and + 8 + {0..3}; rows of tile d were stored with pairs XOR 4 d
+        const u16* vr = &vt[(d * 32 + col) * VROW];
+        const uint2 v0 = *reinterpret_cast<const uint2*>(vr + ((16 * h2 + 4 * half) ^ (8 * d)));
+        const uint2 v1 = *reinterpret_cast<const uint2*>(vr + ((16 * h2 + 8 + 4 * half) ^ (8 * d)));
         const u32x4_t va = {v0.x, v0.y, v1.x, v1.y};
         o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, va), __builtin_bit_cast(bf16x8_t, phi[h2]),
                                                        o[d], 0, 0, 0);
