@@ -355,6 +355,10 @@ __global__ __launch_bounds__(64) void k_attn_prefill(const u16* __restrict__ q, 
 // (p = bf16(p) + bf16(p - bf16(p))), which keeps the fp32 softmax weights to ~2^-17: the result matches
 // the fp32 "math" attention of the eager reference (utils.py:247-258) to rounding of the final bf16.
 // A workgroup is 4 waves = NWH heads of one kv head x NWQ tiles of 32 queries sharing the K / V tiles.
+// e^x through the hardware exp2 (1 ulp in fp32: far below the bf16 rounding of the output); the
+// library expf costs ~15 VALU instructions, and this kernel is VALU-bound next to its MFMAs
+__device__ __forceinline__ float exp_fast(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+
 template <int HD, int NWH>
 __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const u16* __restrict__ q, int64_t ldq,
                                                            const u16* __restrict__ kc, const u16* __restrict__ vc,
@@ -469,12 +473,12 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const u16* __restrict
     float corr = 1.0f;
     u32x4_t phi[2], plo[2];
     if (mn != -INFINITY) {
-      corr = expf(m - mn);  // m == -inf -> 0
+      corr = exp_fast(m - mn);  // m == -inf -> 0
       l *= corr;
       float pv[16];
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        pv[v] = expf(sacc[v] - mn);  // masked -> 0
+        pv[v] = exp_fast(sacc[v] - mn);  // masked -> 0
         l += pv[v];
       }
 #pragma unroll
@@ -495,10 +499,13 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const u16* __restrict
       phi[0] = phi[1] = plo[0] = plo[1] = u32x4_t{0u, 0u, 0u, 0u};
     }
     // ---- O^T += V^T P^T ; k-step h2 covers keys 16 h2 + {0..3, 8..11} + 4 half, in the order of sacc
+    const bool rescale = __any(corr != 1.0f);  // the running maxima rarely move after the first tiles
 #pragma unroll
     for (int d = 0; d < DT; ++d) {
+      if (rescale) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) o[d][v] *= corr;
+        for (int v = 0; v < 16; ++v) o[d][v] *= corr;
+      }
 #pragma unroll
       for (int h2 = 0; h2 < 2; ++h2) {
         // keys 16 h2 + 4 half + {0..3} and + 8 + {0..3}; rows of tile d were stored with pairs XOR 4 d
