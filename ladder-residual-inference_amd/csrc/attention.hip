@@ -69,14 +69,25 @@ __global__ __launch_bounds__(256) void k_attn_decode_partial(const u16* __restri
     return;
   }
 
-  for (int i = tid; i < G * HD; i += 256)
-    qs[i] = bf_to_f(q[(int64_t)b * ldq + (kvh * G + i / HD) * HD + (i % HD)]);
-  __syncthreads();
-
   const int kl = lane / LPK, dl = (lane % LPK) * 8;
   const u16* kbase = kc + ((int64_t)b * Hkv + kvh) * Smax * HD;
   const u16* vbase = vc + ((int64_t)b * Hkv + kvh) * Smax * HD;
   const float scale = rsqrtf((float)HD);
+  // Keys are walked PFB iterations at a time with all loads of a batch requested together, and the
+  // first batch of K and of V is requested before anything else: a 64-key chunk (the usual size)
+  // then costs one memory round trip instead of one per iteration and per operand.
+  constexpr int PFB = 4;
+  const int key00 = k0 + wave * KPW + kl;
+  uint4 kfirst[PFB], vfirst[PFB];
+#pragma unroll
+  for (int u = 0; u < PFB; ++u) {
+    const int key = key00 + u * 4 * KPW;
+    kfirst[u] = key < k1 ? ld16(kbase + (int64_t)key * HD + dl) : make_uint4(0, 0, 0, 0);
+    vfirst[u] = key < k1 ? ld16(vbase + (int64_t)key * HD + dl) : make_uint4(0, 0, 0, 0);
+  }
+  for (int i = tid; i < G * HD; i += 256)
+    qs[i] = bf_to_f(q[(int64_t)b * ldq + (kvh * G + i / HD) * HD + (i % HD)]);
+  __syncthreads();
 
   // ---- scores
   {
@@ -85,18 +96,28 @@ __global__ __launch_bounds__(256) void k_attn_decode_partial(const u16* __restri
     for (int g = 0; g < G; ++g)
 #pragma unroll
       for (int j = 0; j < 8; ++j) qf[g][j] = qs[g * HD + dl + j];
-    for (int key = k0 + wave * KPW + kl; key < k1 + kl; key += 4 * KPW) {  // "+ kl": keep the wave converged
-      const bool live = key < k1;
-      float kf[8];
-      unpack8(live ? ld16(kbase + (int64_t)key * HD + dl) : make_uint4(0, 0, 0, 0), kf);
+    for (int kb = key00; kb < k1 + kl; kb += PFB * 4 * KPW) {  // "+ kl": keep the wave converged
+      uint4 kr[PFB];
 #pragma unroll
-      for (int g = 0; g < G; ++g) {
-        float s = 0.0f;
+      for (int u = 0; u < PFB; ++u) {
+        const int key = kb + u * 4 * KPW;
+        kr[u] = kb == key00 ? kfirst[u] : (key < k1 ? ld16(kbase + (int64_t)key * HD + dl) : make_uint4(0, 0, 0, 0));
+      }
 #pragma unroll
-        for (int j = 0; j < 8; ++j) s = fmaf(kf[j], qf[g][j], s);
+      for (int u = 0; u < PFB; ++u) {
+        const int key = kb + u * 4 * KPW;
+        const bool live = key < k1;
+        float kf[8];
+        unpack8(kr[u], kf);
 #pragma unroll
-        for (int o = 1; o < LPK; o <<= 1) s += __shfl_xor(s, o, LR_WAVE);
-        if (live && (lane % LPK) == 0) sc[g * chunk_max + key - k0] = s * scale;
+        for (int g = 0; g < G; ++g) {
+          float s = 0.0f;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) s = fmaf(kf[j], qf[g][j], s);
+#pragma unroll
+          for (int o = 1; o < LPK; o <<= 1) s += __shfl_xor(s, o, LR_WAVE);
+          if (live && (lane % LPK) == 0) sc[g * chunk_max + key - k0] = s * scale;
+        }
       }
     }
   }
@@ -125,14 +146,26 @@ __global__ __launch_bounds__(256) void k_attn_decode_partial(const u16* __restri
     for (int g = 0; g < G; ++g)
 #pragma unroll
       for (int j = 0; j < 8; ++j) acc[g][j] = 0.0f;
-    for (int key = k0 + wave * KPW + kl; key < k1; key += 4 * KPW) {
-      float vf[8];
-      unpack8(ld16(vbase + (int64_t)key * HD + dl), vf);
+    for (int kb = key00; kb < k1; kb += PFB * 4 * KPW) {
+      uint4 vr[PFB];
 #pragma unroll
-      for (int g = 0; g < G; ++g) {
-        const float p = sc[g * chunk_max + key - k0];
+      for (int u = 0; u < PFB; ++u) {
+        const int key = kb + u * 4 * KPW;
+        vr[u] = kb == key00 ? vfirst[u] : (key < k1 ? ld16(vbase + (int64_t)key * HD + dl) : make_uint4(0, 0, 0, 0));
+      }
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[g][j] = fmaf(p, vf[j], acc[g][j]);
+      for (int u = 0; u < PFB; ++u) {
+        const int key = kb + u * 4 * KPW;
+        if (key < k1) {
+          float vf[8];
+          unpack8(vr[u], vf);
+#pragma unroll
+          for (int g = 0; g < G; ++g) {
+            const float p = sc[g * chunk_max + key - k0];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[g][j] = fmaf(p, vf[j], acc[g][j]);
+          }
+        }
       }
     }
     // fold the KPW key groups of the wave, then the four waves through LDS (fixed order)
