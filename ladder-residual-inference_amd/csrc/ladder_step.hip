@@ -39,7 +39,10 @@
 // "units" (8 rows x 1 KiB of one K-slice) held in two register sets; the set just multiplied is
 // refilled at once with the unit two positions ahead -- also across the end of a job into the
 // next one, through reductions, epilogues, norms and waits -- so a wave has 16 KiB of loads in
-// flight.  The unit sequence of a job is padded to an even length (pad loads go out of the
+// flight.  (One exception: the first units of a slot's first job are requested inside the residual
+// bookkeeping, right after the exchanged words have arrived, not at the end of the previous slot:
+// loads return in order, and those words are what every workgroup is waiting for at that point.)
+// The unit sequence of a job is padded to an even length (pad loads go out of the
 // buffer's range and cost nothing) so that the two sets alternate in a fixed pattern, there is
 // exactly ONE load sequence in the loop, and rows are addressed through a scalar offset from a
 // small per-launch table: that is what lets the compiler place exact wait counts (vmcnt(8))
@@ -681,7 +684,8 @@ constexpr int PRO_NIT = 4;  // 8-element chunks per lane and row: dim <= PRO_NIT
 template <int M>
 __device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, u16* xr, const int* emb_rows,
                                          bool has_d1, unsigned d1_wo, unsigned d1_tag, bool has_d2, unsigned d2_wo,
-                                         unsigned d2_tag, const u16* g1, const u16* g2, u16* x1, u16* x2, float* red) {
+                                         unsigned d2_tag, const u16* g1, const u16* g2, u16* x1, u16* x2, float* red,
+                                         const Job& first, Pipe& pipe) {
   const int tid = opaque_tid(), D = p.D;
   float ss1[M], ss2[M];
   // the gains are needed only in pass 2 but are requested now: their latency hides behind pass 1
@@ -743,6 +747,11 @@ __device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, u1
       }
     }
   }
+  // The first weight units of the coming job are requested only now, behind the exchange words: a
+  // wave's loads return in order and a CU serves them at a bounded rate, so requested at the end of
+  // the previous job they would stand between this phase and the words it waits for; from here they
+  // travel while the norms are finished.
+  prime(first, tid & 63, pipe);
 #pragma unroll
   for (int m = 0; m < M; ++m) {
     ss1[m] = wave_sum(ss1[m]);
@@ -1139,7 +1148,6 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
 
   const int qdim = Hq * HD;
   Pipe pipe;
-  prime(slot_job(p, jtab, lring, 0, 0, wave), lane, pipe);
 
 #define LR_STAMP(k)                                                                                  \
   if (p.prof && t >= p.prof_t0 && t < p.prof_t0 + PROF_SLOTS && tid == 0)                            \
@@ -1156,7 +1164,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
     // ---------------- v1 = R + m(t-2) feeds mlp(t-1); v2 = v1 + a(t-1) feeds attention(t)
     prologue<M>(p, coh, xr, t == 0 ? p.tokens : nullptr, t >= 2, p.om, tag_prev, t >= 1 && has_a, p.oa, tag_prev,
                 has_b ? ring_ptr(lring, t - 1, LP_FFN_NORM) : nullptr,
-                has_a ? ring_ptr(lring, t, LP_ATTN_NORM) : nullptr, xb, xa, red);
+                has_a ? ring_ptr(lring, t, LP_ATTN_NORM) : nullptr, xb, xa, red, LR_JOB(has_a ? 0 : 1), pipe);
     // this workgroup no longer reads a / m / the previous partials
     if (tid == 0) coh.st(p.odone + (unsigned)w, 0.0f, tag);
     LR_STAMP(1)
@@ -1194,7 +1202,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
     if (has_a) {
       attention_merge<M, HD>(p, coh, Hq, tag, xa, wbuf);
       LR_STAMP(4)
-      Job after_wo = next_slot_job(p, jtab, lring, t, wave);
+      Job after_wo = slot_job(p, jtab, lring, -1, 0, wave);
       if (has_b) after_wo = LR_JOB(3);
       run_job<M, EPI_STORE>(p, coh, LR_JOB(2), after_wo, pipe, xa, part, p.oa, D, tag, nullptr, nullptr, nullptr,
                             nullptr);
@@ -1208,7 +1216,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
     if (has_b) {
       load_x<M>(coh, act_wo, tag, I, xb);
       LR_STAMP(6)
-      run_job<M, EPI_STORE>(p, coh, LR_JOB(3), next_slot_job(p, jtab, lring, t, wave), pipe, xb, part, p.om, D, tag,
+      run_job<M, EPI_STORE>(p, coh, LR_JOB(3), slot_job(p, jtab, lring, -1, 0, wave), pipe, xb, part, p.om, D, tag,
                             nullptr, nullptr, nullptr, nullptr);
     }
     LR_STAMP(7)
@@ -1223,7 +1231,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   // ---------------- head: x = (R + a(L-1)) + m(L-1), final norm, vocab-shard lm_head, argmax
   const unsigned tag = tag_of(epoch_base + (unsigned)L + 2u), tag_prev = tag_of(epoch_base + (unsigned)L + 1u);
   prologue<M>(p, coh, xr, nullptr, true, p.oa, tag_of(epoch_base + (unsigned)L), true, p.om, tag_prev, nullptr,
-              p.final_norm, xb, xa, red);
+              p.final_norm, xb, xa, red, slot_job(p, jtab, lring, 4, L + 1, wave), pipe);
   float best_v = -INFINITY;
   int best_i = 0x7fffffff;
   run_job<M, EPI_LOGITS>(p, coh, slot_job(p, jtab, lring, 4, L + 1, wave), slot_job(p, jtab, lring, -1, 0, wave), pipe,
