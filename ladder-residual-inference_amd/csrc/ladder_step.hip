@@ -73,6 +73,7 @@ constexpr int ATT_NI = 9;         // key iterations an attention wave keeps in r
 constexpr int NA_MAX = 16;        // attention workgroups (partial results merged by everyone)
 constexpr int PROF_SLOTS = 4, PROF_POINTS = 12;
 constexpr int AUX_SC1 = 16;       // buffer cache policy: agent scope
+constexpr int AUX_LD = 17;
 
 struct Ctrl {
   unsigned epoch_base, _p0[31];  // slots consumed by earlier steps (tags continue from here)
@@ -172,7 +173,7 @@ struct Coh {
   __device__ __forceinline__ u32x4_t poll4(unsigned wo, unsigned tag) const {
     unsigned spins = 0;
     for (;;) {
-      const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(r, wo * 4, 0, AUX_SC1);
+      const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(r, wo * 4, 0, AUX_LD);
       if ((((a.x ^ tag) | (a.y ^ tag) | (a.z ^ tag) | (a.w ^ tag)) & 0xffffu) == 0) return a;
       if (give_up(spins)) return a;
       __builtin_amdgcn_s_sleep(2);
@@ -181,7 +182,7 @@ struct Coh {
   __device__ __forceinline__ u32x2_t poll2(unsigned wo, unsigned tag) const {
     unsigned spins = 0;
     for (;;) {
-      const u32x2_t a = __builtin_amdgcn_raw_buffer_load_b64(r, wo * 4, 0, AUX_SC1);
+      const u32x2_t a = __builtin_amdgcn_raw_buffer_load_b64(r, wo * 4, 0, AUX_LD);
       if ((((a.x ^ tag) | (a.y ^ tag)) & 0xffffu) == 0) return a;
       if (give_up(spins)) return a;
       __builtin_amdgcn_s_sleep(2);
@@ -190,7 +191,7 @@ struct Coh {
   __device__ __forceinline__ unsigned poll1(unsigned wo, unsigned tag) const {
     unsigned spins = 0;
     for (;;) {
-      const unsigned a = __builtin_amdgcn_raw_buffer_load_b32(r, wo * 4, 0, AUX_SC1);
+      const unsigned a = __builtin_amdgcn_raw_buffer_load_b32(r, wo * 4, 0, AUX_LD);
       if (((a ^ tag) & 0xffffu) == 0) return a;
       if (give_up(spins)) return a;
       __builtin_amdgcn_s_sleep(2);
@@ -199,13 +200,13 @@ struct Coh {
   // Optimistic form: raw4/raw2 issue the load (many can be in flight), settle4/settle2 accept the
   // words if their tags match and fall back to polling otherwise.
   __device__ __forceinline__ u32x4_t raw4(unsigned wo) const {
-    return __builtin_amdgcn_raw_buffer_load_b128(r, wo * 4, 0, AUX_SC1);
+    return __builtin_amdgcn_raw_buffer_load_b128(r, wo * 4, 0, AUX_LD);
   }
   __device__ __forceinline__ unsigned raw1(unsigned wo) const {
-    return __builtin_amdgcn_raw_buffer_load_b32(r, wo * 4, 0, AUX_SC1);
+    return __builtin_amdgcn_raw_buffer_load_b32(r, wo * 4, 0, AUX_LD);
   }
   __device__ __forceinline__ u32x2_t raw2(unsigned wo) const {
-    return __builtin_amdgcn_raw_buffer_load_b64(r, wo * 4, 0, AUX_SC1);
+    return __builtin_amdgcn_raw_buffer_load_b64(r, wo * 4, 0, AUX_LD);
   }
   __device__ __forceinline__ u32x4_t settle4(unsigned wo, unsigned tag, const u32x4_t& a) const {
     if ((((a.x ^ tag) | (a.y ^ tag) | (a.z ^ tag) | (a.w ^ tag)) & 0xffffu) == 0) return a;
@@ -219,8 +220,8 @@ struct Coh {
   __device__ __forceinline__ void ld8(unsigned wo, unsigned tag, float* f) const {
     unsigned spins = 0;
     for (;;) {
-      const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(r, wo * 4, 0, AUX_SC1);
-      const u32x4_t b = __builtin_amdgcn_raw_buffer_load_b128(r, wo * 4 + 16, 0, AUX_SC1);
+      const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(r, wo * 4, 0, AUX_LD);
+      const u32x4_t b = __builtin_amdgcn_raw_buffer_load_b128(r, wo * 4 + 16, 0, AUX_LD);
       const unsigned bad = ((a.x ^ tag) | (a.y ^ tag) | (a.z ^ tag) | (a.w ^ tag) | (b.x ^ tag) | (b.y ^ tag) |
                             (b.z ^ tag) | (b.w ^ tag)) & 0xffffu;
       if (bad == 0 || give_up(spins)) {
