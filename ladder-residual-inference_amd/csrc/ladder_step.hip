@@ -71,9 +71,21 @@ constexpr int RB = 8;  // rows per unit (loads a wave issues together)
 constexpr unsigned SPIN_LIMIT = 1u << 18;
 constexpr int ATT_NI = 9;         // key iterations an attention wave keeps in registers
 constexpr int NA_MAX = 16;        // attention workgroups (partial results merged by everyone)
-constexpr int PROF_SLOTS = 4, PROF_POINTS = 12;
-constexpr int AUX_SC1 = 16;       // buffer cache policy: agent scope
-constexpr int AUX_LD = 17;
+constexpr int PROF_SLOTS = 4, PROF_POINTS = 16;
+#ifndef LR_AUX_ST
+#define LR_AUX_ST 16
+#endif
+#ifndef LR_AUX_LD
+#define LR_AUX_LD 17
+#endif
+#ifndef LR_POLL_SLEEP
+#define LR_POLL_SLEEP 2
+#endif
+constexpr int AUX_SC1 = LR_AUX_ST;       // buffer cache policy: agent scope
+constexpr int AUX_LD = LR_AUX_LD;
+#ifndef LR_W_AUX
+#define LR_W_AUX 2
+#endif
 
 struct Ctrl {
   unsigned epoch_base, _p0[31];  // slots consumed by earlier steps (tags continue from here)
@@ -176,7 +188,7 @@ struct Coh {
       const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(r, wo * 4, 0, AUX_LD);
       if ((((a.x ^ tag) | (a.y ^ tag) | (a.z ^ tag) | (a.w ^ tag)) & 0xffffu) == 0) return a;
       if (give_up(spins)) return a;
-      __builtin_amdgcn_s_sleep(2);
+      __builtin_amdgcn_s_sleep(LR_POLL_SLEEP);
     }
   }
   __device__ __forceinline__ u32x2_t poll2(unsigned wo, unsigned tag) const {
@@ -185,7 +197,7 @@ struct Coh {
       const u32x2_t a = __builtin_amdgcn_raw_buffer_load_b64(r, wo * 4, 0, AUX_LD);
       if ((((a.x ^ tag) | (a.y ^ tag)) & 0xffffu) == 0) return a;
       if (give_up(spins)) return a;
-      __builtin_amdgcn_s_sleep(2);
+      __builtin_amdgcn_s_sleep(LR_POLL_SLEEP);
     }
   }
   __device__ __forceinline__ unsigned poll1(unsigned wo, unsigned tag) const {
@@ -194,7 +206,7 @@ struct Coh {
       const unsigned a = __builtin_amdgcn_raw_buffer_load_b32(r, wo * 4, 0, AUX_LD);
       if (((a ^ tag) & 0xffffu) == 0) return a;
       if (give_up(spins)) return a;
-      __builtin_amdgcn_s_sleep(2);
+      __builtin_amdgcn_s_sleep(LR_POLL_SLEEP);
     }
   }
   // Optimistic form: raw4/raw2 issue the load (many can be in flight), settle4/settle2 accept the
@@ -207,6 +219,9 @@ struct Coh {
   }
   __device__ __forceinline__ u32x2_t raw2(unsigned wo) const {
     return __builtin_amdgcn_raw_buffer_load_b64(r, wo * 4, 0, AUX_LD);
+  }
+  __device__ __forceinline__ bool stale4(const u32x4_t& a, unsigned tag) const {
+    return (((a.x ^ tag) | (a.y ^ tag) | (a.z ^ tag) | (a.w ^ tag)) & 0xffffu) != 0;
   }
   __device__ __forceinline__ u32x4_t settle4(unsigned wo, unsigned tag, const u32x4_t& a) const {
     if ((((a.x ^ tag) | (a.y ^ tag) | (a.z ^ tag) | (a.w ^ tag)) & 0xffffu) == 0) return a;
@@ -231,7 +246,7 @@ struct Coh {
         f[6] = __uint_as_float(b.z & 0xffff0000u); f[7] = __uint_as_float(b.w & 0xffff0000u);
         return;
       }
-      __builtin_amdgcn_s_sleep(2);
+      __builtin_amdgcn_s_sleep(LR_POLL_SLEEP);
     }
   }
   __device__ __forceinline__ void ld2(unsigned wo, unsigned tag, float& x0, float& x1) const {
@@ -466,7 +481,7 @@ __device__ __forceinline__ void load_unit(const Job& job, int j0, int jb, int kk
   }
 #pragma unroll
   for (int i = 0; i < RB; ++i)
-    u.r[i] = __builtin_amdgcn_raw_buffer_load_b128(br, voff, LR_UNI(real ? so[i] : 0), 0);
+    u.r[i] = __builtin_amdgcn_raw_buffer_load_b128(br, voff, LR_UNI(real ? so[i] : 0), LR_W_AUX);
 }
 // ---- a wave's position in the unit sequence of a job.  The sequence is: for every round, the
 //      wave's units (k-steps fastest, then row batches), padded to an even count, so that the two
@@ -686,7 +701,7 @@ template <int M>
 __device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, u16* xr, const int* emb_rows,
                                          bool has_d1, unsigned d1_wo, unsigned d1_tag, bool has_d2, unsigned d2_wo,
                                          unsigned d2_tag, const u16* g1, const u16* g2, u16* x1, u16* x2, float* red,
-                                         const Job& first, Pipe& pipe) {
+                                         const Job& first, Pipe& pipe, unsigned long long* stamp = nullptr) {
   const int tid = opaque_tid(), D = p.D;
   float ss1[M], ss2[M];
   // the gains are needed only in pass 2 but are requested now: their latency hides behind pass 1
@@ -714,6 +729,34 @@ __device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, u1
         r2[it][1] = coh.raw4(d2_wo + m * D + c + 4);
       }
     }
+#ifdef LR_ROUNDS
+    // Words that other workgroups had not written yet are requested again all together, one round
+    // trip per round, instead of one after the other when they are used.
+    for (unsigned spins = 0;;) {
+      unsigned stale = 0;
+#pragma unroll
+      for (int it = 0; it < PRO_NIT; ++it) {
+        const int c = (it * NT + tid) * 8;
+        if (c < D && has_d1) {
+          if (coh.stale4(r1[it][0], d1_tag)) stale |= 1u << (4 * it);
+          if (coh.stale4(r1[it][1], d1_tag)) stale |= 2u << (4 * it);
+        }
+        if (c < D && has_d2) {
+          if (coh.stale4(r2[it][0], d2_tag)) stale |= 4u << (4 * it);
+          if (coh.stale4(r2[it][1], d2_tag)) stale |= 8u << (4 * it);
+        }
+      }
+      if (stale == 0 || coh.give_up(spins)) break;
+#pragma unroll
+      for (int it = 0; it < PRO_NIT; ++it) {
+        const int c = (it * NT + tid) * 8;
+        if (stale & (1u << (4 * it))) r1[it][0] = coh.raw4(d1_wo + m * D + c);
+        if (stale & (2u << (4 * it))) r1[it][1] = coh.raw4(d1_wo + m * D + c + 4);
+        if (stale & (4u << (4 * it))) r2[it][0] = coh.raw4(d2_wo + m * D + c);
+        if (stale & (8u << (4 * it))) r2[it][1] = coh.raw4(d2_wo + m * D + c + 4);
+      }
+    }
+#endif
 #pragma unroll
     for (int it = 0; it < PRO_NIT; ++it) {
       const int c = (it * NT + tid) * 8;
@@ -752,6 +795,7 @@ __device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, u1
   // wave's loads return in order and a CU serves them at a bounded rate, so requested at the end of
   // the previous job they would stand between this phase and the words it waits for; from here they
   // travel while the norms are finished.
+  if (stamp && tid == 0) stamp[12] = wall_clock64();
   prime(first, tid & 63, pipe);
 #pragma unroll
   for (int m = 0; m < M; ++m) {
@@ -766,6 +810,7 @@ __device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, u1
     }
   }
   wg_sync();
+  if (stamp && tid == 0) stamp[13] = wall_clock64();
   // pass 2: scale in place (each lane revisits the elements it wrote)
 #pragma unroll
   for (int m = 0; m < M; ++m) {
@@ -1082,6 +1127,18 @@ __device__ __forceinline__ void attention_merge(const StepParams& p, const Coh& 
       for (int s = 0; s < NA_MAX; ++s)
         if (s < NA) raw[s] = coh.raw4(p.oopart + (unsigned)(((bh * NA + s) * HD + d) * 2));
     }
+#ifdef LR_ROUNDS
+    for (unsigned spins = 0;;) {  // late partials are requested again together, not one by one
+      unsigned stale = 0;
+#pragma unroll
+      for (int s = 0; s < NA_MAX; ++s)
+        if (s < NA && coh.stale4(raw[s], tag)) stale |= 1u << s;
+      if (stale == 0 || coh.give_up(spins)) break;
+#pragma unroll
+      for (int s = 0; s < NA_MAX; ++s)
+        if (stale & (1u << s)) raw[s] = coh.raw4(p.oopart + (unsigned)(((bh * NA + s) * HD + d) * 2));
+    }
+#endif
 #pragma unroll
     for (int s = 0; s < NA_MAX; ++s) {
       if (s < NA) {
@@ -1165,7 +1222,10 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
     // ---------------- v1 = R + m(t-2) feeds mlp(t-1); v2 = v1 + a(t-1) feeds attention(t)
     prologue<M>(p, coh, xr, t == 0 ? p.tokens : nullptr, t >= 2, p.om, tag_prev, t >= 1 && has_a, p.oa, tag_prev,
                 has_b ? ring_ptr(lring, t - 1, LP_FFN_NORM) : nullptr,
-                has_a ? ring_ptr(lring, t, LP_ATTN_NORM) : nullptr, xb, xa, red, LR_JOB(has_a ? 0 : 1), pipe);
+                has_a ? ring_ptr(lring, t, LP_ATTN_NORM) : nullptr, xb, xa, red, LR_JOB(has_a ? 0 : 1), pipe,
+                (p.prof && t >= p.prof_t0 && t < p.prof_t0 + PROF_SLOTS)
+                    ? p.prof + ((size_t)blockIdx.x * PROF_SLOTS + (t - p.prof_t0)) * PROF_POINTS
+                    : nullptr);
     // this workgroup no longer reads a / m / the previous partials
     if (tid == 0) coh.st(p.odone + (unsigned)w, 0.0f, tag);
     LR_STAMP(1)
