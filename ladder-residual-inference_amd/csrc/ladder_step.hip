@@ -112,7 +112,7 @@ struct StepParams {
   int hist_len, pos0, advance;
   unsigned char* ws;  // workspace base (Ctrl at offset 0)
   unsigned ws_bytes;
-  unsigned oa, om, oqkv, oact, oopart, omlpart, ocand, odone;  // exchange buffers, offsets in 32-bit words
+  unsigned oa, om, oqkv, oact, oopart, omlpart, ocand, odone, oy;  // exchange buffers, offsets in 32-bit words
   unsigned long long* prof;  // optional [nwg][PROF_SLOTS][PROF_POINTS] wall-clock stamps (100 MHz)
   int prof_t0;
 };
@@ -165,6 +165,13 @@ struct Coh {
     b.z = (__float_as_uint(f[6]) & 0xffff0000u) | tag; b.w = (__float_as_uint(f[7]) & 0xffff0000u) | tag;
     __builtin_amdgcn_raw_buffer_store_b128(a, r, wo * 4, 0, AUX_SC1);
     __builtin_amdgcn_raw_buffer_store_b128(b, r, wo * 4 + 16, 0, AUX_SC1);
+  }
+  // two bf16-representable values as two words at wo, wo + 1 (wo % 2 == 0)
+  __device__ __forceinline__ void st2(unsigned wo, float v0, float v1, unsigned tag) const {
+    u32x2_t w;
+    w.x = (__float_as_uint(v0) & 0xffff0000u) | tag;
+    w.y = (__float_as_uint(v1) & 0xffff0000u) | tag;
+    __builtin_amdgcn_raw_buffer_store_b64(w, r, wo * 4, 0, AUX_SC1);
   }
   // fp32 value as two words at wo, wo + 1 (wo % 2 == 0)
   __device__ __forceinline__ void st_f32(unsigned wo, float v, unsigned tag) const {
@@ -1154,6 +1161,60 @@ __device__ __forceinline__ void attention_merge(const StepParams& p, const Coh& 
   wg_sync();
 }
 
+// Attention workgroup `aw`: merge the NA partial results for its share of the output pairs and
+// publish them as tagged bf16 words at p.oy ([M][Hq * HD]); everyone else then reads 2 bytes of
+// payload per output element instead of NA fp32 partials.
+template <int M, int HD>
+__device__ __forceinline__ void attention_merge_slice(const StepParams& p, const Coh& coh, int Hq, unsigned tag,
+                                                      float* wbuf, int aw) {
+  const int tid = opaque_tid(), wave = tid >> 6, lane = tid & 63;
+  const int NA = p.NA, nbh = p.B * Hq;
+  const int npairs = nbh * HD / 2;
+  const int per = (npairs + NA - 1) / NA;
+  const int p0 = aw * per, p1 = p0 + per < npairs ? p0 + per : npairs;
+  if (p0 >= p1) return;
+  u32x4_t raw[NA_MAX];
+  {
+    const int pp = p0 + tid;
+    const int bh = (2 * pp) / HD, d = (2 * pp) % HD;
+#pragma unroll
+    for (int s = 0; s < NA_MAX; ++s)
+      raw[s] = (s < NA && pp < p1) ? coh.raw4(p.oopart + (unsigned)(((bh * NA + s) * HD + d) * 2))
+                                   : u32x4_t{0u, 0u, 0u, 0u};
+  }
+  const int bh0 = (2 * p0) / HD, bh1 = (2 * (p1 - 1)) / HD;
+  for (int bh = bh0 + wave; bh <= bh1; bh += NW) {
+    float m = -INFINITY, l = 0.0f;
+    if (lane < NA) f32x2_from(coh.poll4(p.omlpart + (unsigned)((bh * NA + lane) * 4), tag), m, l);
+    const float mx = wave_max(m);
+    const float w = m == -INFINITY ? 0.0f : expf(m - mx);
+    const float L = wave_sum(w * l);
+    if (lane < NA) wbuf[bh * NA_MAX + lane] = L > 0.0f ? w / L : 0.0f;
+  }
+  wg_sync();
+  for (int pp = p0 + tid; pp < p1; pp += NT) {
+    const int bh = (2 * pp) / HD, d = (2 * pp) % HD;
+    float y0 = 0.0f, y1 = 0.0f;
+    if (pp != p0 + tid) {
+#pragma unroll
+      for (int s = 0; s < NA_MAX; ++s)
+        if (s < NA) raw[s] = coh.raw4(p.oopart + (unsigned)(((bh * NA + s) * HD + d) * 2));
+    }
+#pragma unroll
+    for (int s = 0; s < NA_MAX; ++s) {
+      if (s < NA) {
+        float o0, o1;
+        f32x2_from(coh.settle4(p.oopart + (unsigned)(((bh * NA + s) * HD + d) * 2), tag, raw[s]), o0, o1);
+        const float w = wbuf[bh * NA_MAX + s];
+        y0 = fmaf(w, o0, y0);
+        y1 = fmaf(w, o1, y1);
+      }
+    }
+    coh.st2(p.oy + (unsigned)(2 * pp), round_bf(y0), round_bf(y1), tag);
+  }
+  wg_sync();
+}
+
 // ------------------------------------------------------------------------------------------------
 template <int M, int HD, int G>
 __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
@@ -1249,6 +1310,9 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
                                       kv, reinterpret_cast<u32*>(qs), sc, sc_ld, ored, reinterpret_cast<u32*>(knew), vnew, s_m, s_l);
           first = false;
         }
+#ifndef LR_MERGE_ALL
+      attention_merge_slice<M, HD>(p, coh, Hq, tag, wbuf, w);
+#endif
     } else {
       run_job<M, EPI_STORE>(p, coh, LR_JOB(0), LR_JOB(1), pipe, xa, part, p.oqkv, p.nqkv, tag, nullptr, nullptr,
                             nullptr, nullptr);
@@ -1261,7 +1325,11 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
     LR_STAMP(3)
     // ---------------- merge attention partials, output projection
     if (has_a) {
+#ifndef LR_MERGE_ALL
+      load_x<M>(coh, p.oy, tag, qdim, xa);
+#else
       attention_merge<M, HD>(p, coh, Hq, tag, xa, wbuf);
+#endif
       LR_STAMP(4)
       Job after_wo = slot_job(p, jtab, lring, -1, 0, wave);
       if (has_b) after_wo = LR_JOB(3);
@@ -1353,7 +1421,7 @@ __global__ void k_step_init(Ctrl* c, unsigned nwg, unsigned* words, unsigned n_w
 }
 
 struct Layout {
-  size_t ctrl, abuf, mbuf, qkv, act, opart, mlpart, cand, done, total;
+  size_t ctrl, abuf, mbuf, qkv, act, opart, mlpart, cand, done, y, total;
 };
 
 static int num_cus() {
@@ -1403,6 +1471,7 @@ static Layout make_layout(const lr_ladder_model_t* md, int B, int nwg) {
   l.mlpart = o; o = up(o + 4 * (size_t)B * Hq * na * 4);
   l.cand = o; o = up(o + 4 * (size_t)nwg * B * 4);
   l.done = o; o = up(o + 4 * (size_t)nwg);
+  l.y = o; o = up(o + 4 * (size_t)B * Hq * hd);
   l.total = o;
   return l;
 }
@@ -1532,7 +1601,7 @@ extern "C" int lr_ladder_decode_step(const lr_ladder_model_t* md, int batch, con
   sp.oa = (unsigned)(l.abuf / 4); sp.om = (unsigned)(l.mbuf / 4);
   sp.oqkv = (unsigned)(l.qkv / 4); sp.oact = (unsigned)(l.act / 4);
   sp.oopart = (unsigned)(l.opart / 4); sp.omlpart = (unsigned)(l.mlpart / 4); sp.ocand = (unsigned)(l.cand / 4);
-  sp.odone = (unsigned)(l.done / 4);
+  sp.odone = (unsigned)(l.done / 4); sp.oy = (unsigned)(l.y / 4);
   sp.prof = g_prof;
   sp.prof_t0 = g_prof_t0;
   hipStream_t s = (hipStream_t)stream;
