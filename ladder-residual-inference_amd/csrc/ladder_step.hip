@@ -703,12 +703,18 @@ __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, con
 // arrays; all their loads are issued before the first one is checked.
 // ------------------------------------------------------------------------------------------------
 constexpr int PRO_NIT = 4;  // 8-element chunks per lane and row: dim <= PRO_NIT * NT * 8
+template <int M>
+struct LateNorm {  // what is needed to finish x1 after the phase that uses x2 (see prologue, finish_x1)
+  uint4 g[PRO_NIT];
+  float inv[M];
+};
 
 template <int M>
 __device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, u16* xr, const int* emb_rows,
                                          bool has_d1, unsigned d1_wo, unsigned d1_tag, bool has_d2, unsigned d2_wo,
                                          unsigned d2_tag, const u16* g1, const u16* g2, u16* x1, u16* x2, float* red,
-                                         const Job& first, Pipe& pipe, unsigned long long* stamp = nullptr) {
+                                         const Job& first, Pipe& pipe, unsigned long long* stamp, LateNorm<M>& late,
+                                         bool defer1) {
   const int tid = opaque_tid(), D = p.D;
   float ss1[M], ss2[M];
   // the gains are needed only in pass 2 but are requested now: their latency hides behind pass 1
@@ -828,12 +834,13 @@ __device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, u1
       s2 += red[(wv * M + m) * 2 + 1];
     }
     const float inv1 = rsqrtf(s1 / (float)D + p.eps), inv2 = rsqrtf(s2 / (float)D + p.eps);
+    late.inv[m] = inv1;
 #pragma unroll
     for (int it = 0; it < PRO_NIT; ++it) {
       const int c = (it * NT + tid) * 8;
       if (c >= D) break;
       float v[8], g[8], o[8];
-      if (g1) {
+      if (g1 && !defer1) {
         unpack8(*reinterpret_cast<const uint4*>(x1 + m * D + c), v);
         unpack8(gq1[it], g);
 #pragma unroll
@@ -847,6 +854,30 @@ __device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, u1
         for (int j = 0; j < 8; ++j) o[j] = round_bf(v[j] * inv2) * g[j];
         st16(x2 + m * D + c, pack8(o));
       }
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < PRO_NIT; ++it) late.g[it] = gq1[it];
+  wg_sync();
+}
+
+// The scaling of x1 that prologue() left out (defer1): x1 = round(v1 * inv) * g1, in place.  Only
+// the workgroups that use x1 call it, after the phase that needed x2 first.
+template <int M>
+__device__ __forceinline__ void finish_x1(const StepParams& p, u16* x1, const LateNorm<M>& late) {
+  const int tid = opaque_tid(), D = p.D;
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+#pragma unroll
+    for (int it = 0; it < PRO_NIT; ++it) {
+      const int c = (it * NT + tid) * 8;
+      if (c >= D) break;
+      float v[8], g[8], o[8];
+      unpack8(*reinterpret_cast<const uint4*>(x1 + m * D + c), v);
+      unpack8(late.g[it], g);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = round_bf(v[j] * late.inv[m]) * g[j];
+      st16(x1 + m * D + c, pack8(o));
     }
   }
   wg_sync();
@@ -1267,6 +1298,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
 
   const int qdim = Hq * HD;
   Pipe pipe;
+  LateNorm<M> late;
 
 #define LR_STAMP(k)                                                                                  \
   if (p.prof && t >= p.prof_t0 && t < p.prof_t0 + PROF_SLOTS && tid == 0)                            \
@@ -1286,7 +1318,8 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
                 has_a ? ring_ptr(lring, t, LP_ATTN_NORM) : nullptr, xb, xa, red, LR_JOB(has_a ? 0 : 1), pipe,
                 (p.prof && t >= p.prof_t0 && t < p.prof_t0 + PROF_SLOTS)
                     ? p.prof + ((size_t)blockIdx.x * PROF_SLOTS + (t - p.prof_t0)) * PROF_POINTS
-                    : nullptr);
+                    : nullptr,
+                late, has_a && has_b);
     // this workgroup no longer reads a / m / the previous partials
     if (tid == 0) coh.st(p.odone + (unsigned)w, 0.0f, tag);
     LR_STAMP(1)
@@ -1317,6 +1350,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
       run_job<M, EPI_STORE>(p, coh, LR_JOB(0), LR_JOB(1), pipe, xa, part, p.oqkv, p.nqkv, tag, nullptr, nullptr,
                             nullptr, nullptr);
       LR_STAMP(2)
+      if (has_a && has_b) finish_x1<M>(p, xb, late);  // its first weight units are on their way meanwhile
       // ---------------- everyone else: the up/gate projection of the previous layer + SwiGLU
       const Job after_w1 = LR_JOB(has_a ? 2 : 3);  // named values, not conditional temporaries: they stay in registers
       run_job<M, EPI_SWIGLU>(p, coh, LR_JOB(1), after_w1, pipe, xb, part, act_wo, I, tag, nullptr, nullptr, nullptr,
@@ -1360,7 +1394,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   // ---------------- head: x = (R + a(L-1)) + m(L-1), final norm, vocab-shard lm_head, argmax
   const unsigned tag = tag_of(epoch_base + (unsigned)L + 2u), tag_prev = tag_of(epoch_base + (unsigned)L + 1u);
   prologue<M>(p, coh, xr, nullptr, true, p.oa, tag_of(epoch_base + (unsigned)L), true, p.om, tag_prev, nullptr,
-              p.final_norm, xb, xa, red, slot_job(p, jtab, lring, 4, L + 1, wave), pipe);
+              p.final_norm, xb, xa, red, slot_job(p, jtab, lring, 4, L + 1, wave), pipe, nullptr, late, false);
   float best_v = -INFINITY;
   int best_i = 0x7fffffff;
   run_job<M, EPI_LOGITS>(p, coh, slot_job(p, jtab, lring, 4, L + 1, wave), slot_job(p, jtab, lring, -1, 0, wave), pipe,
