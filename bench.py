@@ -35,7 +35,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes one k_ladder_step launch moves on the headline workload, from the rocprofv3 counter runs
 # summarised under profiles/ (None until measured).
-TRAFFIC_BYTES_PER_LAUNCH = 17.849e9  # B=1, prompt 2048; 1.022 x algorithmic
+TRAFFIC_BYTES_PER_LAUNCH = 17.692e9  # B=1, prompt 2048; 1.013 x algorithmic
 
 
 def cpu_baseline(new_tokens=32, repeats=2):
