@@ -151,6 +151,17 @@ def test_tiny_ladder_fused_head_dim_128_many_kv_heads():
     assert stats["fused_step_used"]
 
 
+@pytest.mark.parametrize("B", [1, 2])
+def test_fused_step_several_attention_workgroups_ragged_merge_shares(B):
+    # a cache of 360 slots gives three attention workgroups; 8 heads x 64 / 2 = 256 (B = 1) or 512 output pairs
+    # are merged in shares of 86, 86, 84 (171, 171, 170) by the attention workgroups; the key range splits unevenly
+    kw = dict(TINY, block_size=360, n_head=8, n_local_heads=2, dim=512, intermediate_size=640, n_layer=3)
+    stats = run_parity(build("ladder", **kw), "ladder", B=B, T=330, new=10, fused=True)
+    print(B, stats)
+    check(stats)
+    assert stats["fused_step_used"]
+
+
 @pytest.mark.parametrize("family", ["ladder", "dense", "desync", "parallel"])
 @pytest.mark.parametrize("B", [1, 3])
 def test_tiny_all_families(family, B):
