@@ -14,16 +14,19 @@
 //     wqkv(t) rows
 //     attention workgroups (about one per 128 keys): attention(t) over their key range with K/V
 //         held in registers -- scores on the matrix cores (v_mfma_f32_32x32x16_bf16, one tile per
-//         32 keys), fp32 softmax and P.V -- un-normalised partial results
-//     all other workgroups: w1(t-1) rows + SwiGLU  (17 us of streaming that hides the attention
-//         latency chain)
-//     merge the partial results, wo(t) rows
+//         32 keys), fp32 softmax and P.V -- un-normalised partial results; then each of them
+//         merges all partial results for its share of the output elements and publishes bf16
+//         words (every workgroup merging every partial itself costs 32 times the coherent reads,
+//         and those are what makes stragglers)
+//     all other workgroups: the scaling of the MLP input, left out of the norms above, then
+//         w1(t-1) rows + SwiGLU  (17 us of streaming that hides the attention latency chain)
+//     read the merged attention output, wo(t) rows
 //     w2(t-1) rows
 //
 // No barriers, flags or fences: everything that crosses workgroups (module outputs a / m, qkv,
 // activations, attention partials, argmax candidates) is exchanged as self-validating 32-bit
 // words -- 16 payload bits plus the 16-bit tag of the slot that produced them -- written and read
-// with buffer instructions carrying the sc1 (agent-coherent) policy, which bypass the
+// with buffer instructions carrying the sc1 policy (loads: sc0 sc1), which bypass the
 // non-coherent per-XCD L2 lines.  A consumer optimistically loads what it needs and retries the
 // words whose tag is not yet the expected one, so a value is consumed the moment it lands and a
 // producer never waits.  Overwriting a word is safe once every workgroup has finished reading its
@@ -46,7 +49,9 @@
 // buffer's range and cost nothing) so that the two sets alternate in a fixed pattern, there is
 // exactly ONE load sequence in the loop, and rows are addressed through a scalar offset from a
 // small per-launch table: that is what lets the compiler place exact wait counts (vmcnt(8))
-// instead of draining the pipeline.  The multiply is v_dot2_f32_bf16 on packed bf16 pairs.  GEMV
+// instead of draining the pipeline.  Weight loads carry the non-temporal hint: each byte is used
+// once per step and must not push the exchanged words out of the caches.  The multiply is
+// v_dot2_f32_bf16 on packed bf16 pairs.  GEMV
 // rows are dealt to workgroups round-robin so that the CUs working at the same time read
 // neighbouring rows (HBM-channel friendly); inside a workgroup the waves split K, partial sums
 // meet in LDS in a fixed order -- no float atomics, bit-reproducible.  Workgroup barriers wait for
@@ -70,22 +75,13 @@ constexpr int NJMAX = 64;         // GEMV rows a workgroup reduces per LDS round
 constexpr int RB = 8;  // rows per unit (loads a wave issues together)
 constexpr unsigned SPIN_LIMIT = 1u << 18;
 constexpr int ATT_NI = 9;         // key iterations an attention wave keeps in registers
-constexpr int NA_MAX = 16;        // attention workgroups (partial results merged by everyone)
+constexpr int NA_MAX = 16;        // attention workgroups (each merges a share of the outputs)
 constexpr int PROF_SLOTS = 4, PROF_POINTS = 16;
-#ifndef LR_AUX_ST
-#define LR_AUX_ST 16
-#endif
-#ifndef LR_AUX_LD
-#define LR_AUX_LD 17
-#endif
-#ifndef LR_POLL_SLEEP
-#define LR_POLL_SLEEP 2
-#endif
-constexpr int AUX_SC1 = LR_AUX_ST;       // buffer cache policy: agent scope
-constexpr int AUX_LD = LR_AUX_LD;
-#ifndef LR_W_AUX
-#define LR_W_AUX 2
-#endif
+// Buffer cache policies (the `aux` operand of the raw buffer builtins: bit 0 sc0, bit 1 nt, bit 4 sc1).
+constexpr int AUX_SC1 = 16;  // exchange stores: written through, visible to every XCD
+constexpr int AUX_LD = 17;   // exchange loads: sc0 sc1, never served from a per-XCD L2 line
+constexpr int AUX_W = 2;     // weight loads: non-temporal (measured: nt on the exchange words' loads or stores is far slower)
+constexpr int POLL_SLEEP = 2;
 
 struct Ctrl {
   unsigned epoch_base, _p0[31];  // slots consumed by earlier steps (tags continue from here)
@@ -195,7 +191,7 @@ struct Coh {
       const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(r, wo * 4, 0, AUX_LD);
       if ((((a.x ^ tag) | (a.y ^ tag) | (a.z ^ tag) | (a.w ^ tag)) & 0xffffu) == 0) return a;
       if (give_up(spins)) return a;
-      __builtin_amdgcn_s_sleep(LR_POLL_SLEEP);
+      __builtin_amdgcn_s_sleep(POLL_SLEEP);
     }
   }
   __device__ __forceinline__ u32x2_t poll2(unsigned wo, unsigned tag) const {
@@ -204,7 +200,7 @@ struct Coh {
       const u32x2_t a = __builtin_amdgcn_raw_buffer_load_b64(r, wo * 4, 0, AUX_LD);
       if ((((a.x ^ tag) | (a.y ^ tag)) & 0xffffu) == 0) return a;
       if (give_up(spins)) return a;
-      __builtin_amdgcn_s_sleep(LR_POLL_SLEEP);
+      __builtin_amdgcn_s_sleep(POLL_SLEEP);
     }
   }
   __device__ __forceinline__ unsigned poll1(unsigned wo, unsigned tag) const {
@@ -213,7 +209,7 @@ struct Coh {
       const unsigned a = __builtin_amdgcn_raw_buffer_load_b32(r, wo * 4, 0, AUX_LD);
       if (((a ^ tag) & 0xffffu) == 0) return a;
       if (give_up(spins)) return a;
-      __builtin_amdgcn_s_sleep(LR_POLL_SLEEP);
+      __builtin_amdgcn_s_sleep(POLL_SLEEP);
     }
   }
   // Optimistic form: raw4/raw2 issue the load (many can be in flight), settle4/settle2 accept the
@@ -253,7 +249,7 @@ struct Coh {
         f[6] = __uint_as_float(b.z & 0xffff0000u); f[7] = __uint_as_float(b.w & 0xffff0000u);
         return;
       }
-      __builtin_amdgcn_s_sleep(LR_POLL_SLEEP);
+      __builtin_amdgcn_s_sleep(POLL_SLEEP);
     }
   }
   __device__ __forceinline__ void ld2(unsigned wo, unsigned tag, float& x0, float& x1) const {
@@ -488,7 +484,7 @@ __device__ __forceinline__ void load_unit(const Job& job, int j0, int jb, int kk
   }
 #pragma unroll
   for (int i = 0; i < RB; ++i)
-    u.r[i] = __builtin_amdgcn_raw_buffer_load_b128(br, voff, LR_UNI(real ? so[i] : 0), LR_W_AUX);
+    u.r[i] = __builtin_amdgcn_raw_buffer_load_b128(br, voff, LR_UNI(real ? so[i] : 0), AUX_W);
 }
 // ---- a wave's position in the unit sequence of a job.  The sequence is: for every round, the
 //      wave's units (k-steps fastest, then row batches), padded to an even count, so that the two
@@ -742,34 +738,6 @@ __device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, u1
         r2[it][1] = coh.raw4(d2_wo + m * D + c + 4);
       }
     }
-#ifdef LR_ROUNDS
-    // Words that other workgroups had not written yet are requested again all together, one round
-    // trip per round, instead of one after the other when they are used.
-    for (unsigned spins = 0;;) {
-      unsigned stale = 0;
-#pragma unroll
-      for (int it = 0; it < PRO_NIT; ++it) {
-        const int c = (it * NT + tid) * 8;
-        if (c < D && has_d1) {
-          if (coh.stale4(r1[it][0], d1_tag)) stale |= 1u << (4 * it);
-          if (coh.stale4(r1[it][1], d1_tag)) stale |= 2u << (4 * it);
-        }
-        if (c < D && has_d2) {
-          if (coh.stale4(r2[it][0], d2_tag)) stale |= 4u << (4 * it);
-          if (coh.stale4(r2[it][1], d2_tag)) stale |= 8u << (4 * it);
-        }
-      }
-      if (stale == 0 || coh.give_up(spins)) break;
-#pragma unroll
-      for (int it = 0; it < PRO_NIT; ++it) {
-        const int c = (it * NT + tid) * 8;
-        if (stale & (1u << (4 * it))) r1[it][0] = coh.raw4(d1_wo + m * D + c);
-        if (stale & (2u << (4 * it))) r1[it][1] = coh.raw4(d1_wo + m * D + c + 4);
-        if (stale & (4u << (4 * it))) r2[it][0] = coh.raw4(d2_wo + m * D + c);
-        if (stale & (8u << (4 * it))) r2[it][1] = coh.raw4(d2_wo + m * D + c + 4);
-      }
-    }
-#endif
 #pragma unroll
     for (int it = 0; it < PRO_NIT; ++it) {
       const int c = (it * NT + tid) * 8;
@@ -1130,70 +1098,9 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
   wg_sync();
 }
 
-// Every workgroup: merge the NA partial attention results into y [M][Hq * HD] (bf16, LDS).
-//   y = sum_s w_s o_s,  w_s = exp(m_s - max) / sum_s' exp(m_s' - max) l_s'
-template <int M, int HD>
-__device__ __forceinline__ void attention_merge(const StepParams& p, const Coh& coh, int Hq, unsigned tag, u16* y,
-                                                float* wbuf) {
-  const int tid = opaque_tid(), wave = tid >> 6, lane = tid & 63;
-  const int NA = p.NA, nbh = p.B * Hq;
-  const int npairs = nbh * HD / 2;
-  // the partial outputs of this lane's first pair are requested before the weights are worked out
-  u32x4_t raw[NA_MAX];
-  {
-    const int bh = (2 * tid) / HD, d = (2 * tid) % HD;
-#pragma unroll
-    for (int s = 0; s < NA_MAX; ++s)
-      raw[s] = (s < NA && tid < npairs) ? coh.raw4(p.oopart + (unsigned)(((bh * NA + s) * HD + d) * 2))
-                                        : u32x4_t{0u, 0u, 0u, 0u};
-  }
-  // weights: a wave per (sequence, head); lanes < NA hold one chunk each
-  for (int bh = wave; bh < nbh; bh += NW) {
-    float m = -INFINITY, l = 0.0f;
-    if (lane < NA) f32x2_from(coh.poll4(p.omlpart + (unsigned)((bh * NA + lane) * 4), tag), m, l);
-    const float mx = wave_max(m);
-    const float w = m == -INFINITY ? 0.0f : expf(m - mx);
-    const float L = wave_sum(w * l);
-    if (lane < NA) wbuf[bh * NA_MAX + lane] = L > 0.0f ? w / L : 0.0f;
-  }
-  wg_sync();
-  for (int pp = tid; pp < npairs; pp += NT) {
-    const int bh = (2 * pp) / HD, d = (2 * pp) % HD;
-    float y0 = 0.0f, y1 = 0.0f;
-    if (pp != tid) {
-#pragma unroll
-      for (int s = 0; s < NA_MAX; ++s)
-        if (s < NA) raw[s] = coh.raw4(p.oopart + (unsigned)(((bh * NA + s) * HD + d) * 2));
-    }
-#ifdef LR_ROUNDS
-    for (unsigned spins = 0;;) {  // late partials are requested again together, not one by one
-      unsigned stale = 0;
-#pragma unroll
-      for (int s = 0; s < NA_MAX; ++s)
-        if (s < NA && coh.stale4(raw[s], tag)) stale |= 1u << s;
-      if (stale == 0 || coh.give_up(spins)) break;
-#pragma unroll
-      for (int s = 0; s < NA_MAX; ++s)
-        if (stale & (1u << s)) raw[s] = coh.raw4(p.oopart + (unsigned)(((bh * NA + s) * HD + d) * 2));
-    }
-#endif
-#pragma unroll
-    for (int s = 0; s < NA_MAX; ++s) {
-      if (s < NA) {
-        float o0, o1;
-        f32x2_from(coh.settle4(p.oopart + (unsigned)(((bh * NA + s) * HD + d) * 2), tag, raw[s]), o0, o1);
-        const float w = wbuf[bh * NA_MAX + s];
-        y0 = fmaf(w, o0, y0);
-        y1 = fmaf(w, o1, y1);
-      }
-    }
-    *reinterpret_cast<u32*>(y + 2 * pp) = pack_bf2(y0, y1);
-  }
-  wg_sync();
-}
-
-// Attention workgroup `aw`: merge the NA partial results for its share of the output pairs and
-// publish them as tagged bf16 words at p.oy ([M][Hq * HD]); everyone else then reads 2 bytes of
+// Attention workgroup `aw`: merge the NA partial results for its share of the output pairs,
+//   y = sum_s w_s o_s,  w_s = exp(m_s - max) / sum_s' exp(m_s' - max) l_s',
+// and publish them as tagged bf16 words at p.oy ([M][Hq * HD]); everyone else then reads 2 bytes of
 // payload per output element instead of NA fp32 partials.
 template <int M, int HD>
 __device__ __forceinline__ void attention_merge_slice(const StepParams& p, const Coh& coh, int Hq, unsigned tag,
@@ -1343,9 +1250,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
                                       kv, reinterpret_cast<u32*>(qs), sc, sc_ld, ored, reinterpret_cast<u32*>(knew), vnew, s_m, s_l);
           first = false;
         }
-#ifndef LR_MERGE_ALL
       attention_merge_slice<M, HD>(p, coh, Hq, tag, wbuf, w);
-#endif
     } else {
       run_job<M, EPI_STORE>(p, coh, LR_JOB(0), LR_JOB(1), pipe, xa, part, p.oqkv, p.nqkv, tag, nullptr, nullptr,
                             nullptr, nullptr);
@@ -1357,13 +1262,9 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
                              nullptr);
     }
     LR_STAMP(3)
-    // ---------------- merge attention partials, output projection
+    // ---------------- merged attention output (published by the attention workgroups), output projection
     if (has_a) {
-#ifndef LR_MERGE_ALL
       load_x<M>(coh, p.oy, tag, qdim, xa);
-#else
-      attention_merge<M, HD>(p, coh, Hq, tag, xa, wbuf);
-#endif
       LR_STAMP(4)
       Job after_wo = slot_job(p, jtab, lring, -1, 0, wave);
       if (has_b) after_wo = LR_JOB(3);
