@@ -162,6 +162,31 @@ def test_fused_step_several_attention_workgroups_ragged_merge_shares(B):
     assert stats["fused_step_used"]
 
 
+@torch.no_grad()
+def test_fused_step_exchange_tags_wrap_around():
+    # every exchanged word carries a 16-bit tag of the slot that wrote it; a 3-layer step uses 5 tags, so 65535 tags
+    # are used up after 13107 launches.  The step is deterministic: the same token at the same position must give
+    # the same logits, bit for bit, before the wrap, across it and after it, and no wait may time out.
+    model = build("ladder", **TINY)
+    model.use_fused_step = True
+    T = 20
+    model.setup_caches(1, T + 4)
+    g = torch.Generator(device=DEV)
+    g.manual_seed(3)
+    prompt = torch.randint(0, TINY["vocab_size"], (1, T), device=DEV, generator=g)
+    model(prompt, torch.arange(T, device=DEV))
+    tok = torch.tensor([[7]], dtype=torch.int32, device=DEV)
+    pos = torch.tensor([T], dtype=torch.int32, device=DEV)
+    first = model(tok, pos).clone()
+    fs = model._fused[1]
+    for i in range(13400):
+        out = model(tok, pos)
+        if i in (13000, 13100, 13110, 13399):
+            assert torch.equal(out, first), i
+    torch.cuda.synchronize()
+    assert not fs.failed()
+
+
 @pytest.mark.parametrize("family", ["ladder", "dense", "desync", "parallel"])
 @pytest.mark.parametrize("B", [1, 3])
 def test_tiny_all_families(family, B):
