@@ -17,6 +17,9 @@ Prints ONE JSON line.  `value` = decoded tokens per second (whole job = the one 
                launch stream.  `traffic` = HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE
                counter runs (a constant recorded from those runs, or null).  Other models / batches
                fall back to the per-op path, whose dominant kernel is the w1 GEMV.
+               `measured_read_ceiling` = GB/s of a plain streaming read of 8 GiB by every CU
+               (lr_stream_read) on this machine in the same run; `frac` is against the nominal
+               8 TB/s, `frac_of_measured_ceiling` against that.
 `step_roofline`: the same ratio for the whole decode step as replayed from the hipGraph (kernel +
                token hand-over): algorithmic bytes per step / measured step time.
 `cpu_baseline`: the oracle (a PyTorch-CPU restatement of the reference; the reference itself cannot
@@ -185,6 +188,21 @@ def main():
         k_name = f"k_gemv (w1 up+gate projection, [{N} x {Kdim}] bf16, M={B})"
     k_gbps = k_bytes / (k_us * 1e-6) / 1e9
 
+    # ---- the read rate this machine reaches: a plain streaming read of 8 GiB by every CU
+    ceil_buf = torch.empty(8 << 30, dtype=torch.uint8, device=dev)
+    ceil_buf.view(torch.int32).fill_(0x01010101)
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    for _ in range(2):
+        _hip.stream_read(ceil_buf, sink)
+    torch.cuda.synchronize()
+    ev0.record()
+    for _ in range(5):
+        _hip.stream_read(ceil_buf, sink)
+    ev1.record()
+    torch.cuda.synchronize()
+    ceiling_gbps = 5 * ceil_buf.numel() / (ev0.elapsed_time(ev1) * 1e-3) / 1e9
+    del ceil_buf
+
     out = {
         "metric": "decode_tokens_per_sec", "value": round(B * 1e3 / ms_per_step, 2), "unit": "tok/s",
         "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
@@ -199,7 +217,9 @@ def main():
         "roofline": {"bound": "hbm", "kernel": k_name,
                      "achieved": round(k_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(k_gbps / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH if fused else None,
-                     "bytes_per_launch": int(k_bytes), "avg_launch_us": round(k_us, 3)},
+                     "bytes_per_launch": int(k_bytes), "avg_launch_us": round(k_us, 3),
+                     "measured_read_ceiling": round(ceiling_gbps, 1),
+                     "frac_of_measured_ceiling": round(k_gbps / ceiling_gbps, 4)},
         "step_roofline": {"bound": "hbm", "achieved": round(step_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                           "frac": round(step_gbps / HBM_PEAK_GBPS, 4), "bytes_per_step": int(step_bytes)},
         "first_tokens": tokens,

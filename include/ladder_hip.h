@@ -118,6 +118,13 @@ int lr_attn_prefill(const void* q, int64_t ldq, const void* k_cache, const void*
  * out int32 [B].  Greedy stand-in for sample() (benchmark.py:73-77): torch.argmax(logits[:, -1]). */
 int lr_argmax(const void* logits, int64_t ldl, int32_t* out, int B, int V, lr_stream_t stream);
 
+/* Measurement aid, no counterpart in the reference: reads `bytes` of device memory at `src` once
+ * with every CU streaming (16-byte non-temporal loads, nothing written unless the xor of the data
+ * has one particular value, then one word at `sink`).  bench.py times it to report the read rate
+ * this machine reaches beside the nominal HBM peak.  bytes >= 32 KiB; the tail beyond a multiple
+ * of 32 KiB per workgroup round may be left unread. */
+int lr_stream_read(const void* src, size_t bytes, uint32_t* sink, lr_stream_t stream);
+
 /* Device-side bookkeeping between two decode steps, what generate_using_cuda_graphs does on the
  * host between replays (benchmark.py:208-217):
  *     if (history) history[b, pos[0] - pos0] = next_token[b]     (slots outside [0, hist_len) skipped)

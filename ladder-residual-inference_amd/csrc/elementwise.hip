@@ -322,3 +322,33 @@ extern "C" const char* lr_error_string(int code) {
     default: return "unknown error code";
   }
 }
+
+// ------------------------------------------------------------------------------------ stream read
+// Plain streaming read of a buffer by the whole chip: 8 workgroups per CU, 8 x 16 bytes in flight
+// per lane, consecutive workgroups on consecutive 32 KiB blocks, non-temporal loads.  The rate it
+// reaches is the read ceiling of the machine the benchmark runs on, reported beside the nominal
+// HBM peak.  The xor of everything read goes to `sink` only if it has one impossible value, so the
+// loads cannot be dropped.
+__global__ __launch_bounds__(256) void k_stream_read(const u32x4_t* __restrict__ p, size_t n16, unsigned* sink) {
+  constexpr int U = 8;
+  unsigned acc = 0;
+  const size_t stride = (size_t)gridDim.x * 256 * U;
+  for (size_t i = (size_t)blockIdx.x * 256 * U + threadIdx.x; i + (U - 1) * 256 < n16; i += stride) {
+    u32x4_t v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(p + i + u * 256);
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+  }
+  if (acc == 0x9e3779b9u) sink[0] = acc;
+}
+
+extern "C" int lr_stream_read(const void* src, size_t bytes, uint32_t* sink, lr_stream_t stream) {
+  LR_REQUIRE_PTR(src);
+  if (sink == nullptr) return LR_E_NULL;
+  if (bytes < (size_t)256 * 8 * 16) return LR_E_SHAPE;
+  int dev = 0, cus = 256;
+  if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  k_stream_read<<<dim3(cus * 8), dim3(256), 0, (hipStream_t)stream>>>((const u32x4_t*)src, bytes / 16, sink);
+  return lr_launch_status();
+}

@@ -30,6 +30,7 @@ _PROTOS = {
     "lr_attn_prefill": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,
                                 c_int, c_int, c_int, c_int, c_void_p]),
     "lr_argmax": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_int, c_void_p]),
+    "lr_stream_read": (c_int, [c_void_p, c_size_t, c_void_p, c_void_p]),
     "lr_sample_topk": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_float, c_int, c_void_p, c_int64,
                                c_void_p, c_void_p]),
     "lr_advance": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_void_p]),
@@ -205,6 +206,13 @@ def attn_prefill(q, k_cache, v_cache, pos, y, B, S, Hq, Hkv, hd):
     _check(load().lr_attn_prefill(_dev(q), ldq, _dev(k_cache), _dev(v_cache), pos.data_ptr(), _dev(y), ldy, B, S, Hq,
                                   Hkv, hd, Smax, _stream()), "lr_attn_prefill")
     return y
+
+
+def stream_read(buf: torch.Tensor, sink: torch.Tensor):
+    """One streaming read of `buf` by the whole GPU (measurement aid: the machine's read ceiling)."""
+    assert buf.is_cuda and buf.is_contiguous() and sink.is_cuda and sink.dtype == torch.int32
+    _check(load().lr_stream_read(buf.data_ptr(), buf.numel() * buf.element_size(), sink.data_ptr(), _stream()),
+           "lr_stream_read")
 
 
 def argmax(logits: torch.Tensor, out: torch.Tensor):

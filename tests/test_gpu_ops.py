@@ -320,3 +320,17 @@ def test_torch_argmax_itself_returns_first_maximum_on_this_device():
     lg = torch.zeros(1, 16032, dtype=BF, device=DEV)
     lg[0, [15000, 40, 9000]] = 1.0
     assert torch.argmax(lg, -1).item() == 40
+
+
+# ------------------------------------------------------------------------------------ stream read
+
+def test_stream_read_runs_and_leaves_the_sink_alone(hip):
+    """The measurement aid reads the buffer and writes nothing (the xor of the data is not the magic value)."""
+    buf = torch.full((64 << 20,), 3, dtype=torch.uint8, device=DEV)
+    sink = torch.full((1,), 1234, dtype=torch.int32, device=DEV)
+    for _ in range(3):
+        hip.stream_read(buf, sink)
+    torch.cuda.synchronize()
+    assert sink.item() == 1234
+    with pytest.raises(hip.LadderHipError):
+        hip.stream_read(buf[:1024], sink)
