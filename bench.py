@@ -139,6 +139,7 @@ def main():
         dg.replay()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    model.check_device_errors()   # raises if any timed step did not do its work (expired wait, position out of range)
     ms_per_step = 1e3 * elapsed / K
     tokens = dg.history[0, : min(K, 16)].tolist()
 
@@ -163,6 +164,7 @@ def main():
         ev1.record()
         torch.cuda.synchronize()
         k_us = 1e3 * ev0.elapsed_time(ev1) / reps
+        model.check_device_errors()
         k_bytes = bm.decode_bytes_per_step(cfg, B, T)
         k_name = (f"k_ladder_step (one persistent launch = the whole decode step at position {T}: "
                   f"{cfg.n_layer} layers + lm_head, M={B})")

@@ -41,6 +41,14 @@ enum {
   LR_E_LAUNCH = -5       /* the HIP runtime refused the launch                            */
 };
 
+/* Values of device-side error words (lr_rope_kv_write's `err`, the workspace word at
+ * lr_ladder_step_fail_offset()): conditions only the device can see, reported without a host
+ * synchronisation.  0 = none. */
+enum {
+  LR_DEV_WAIT_EXPIRED = 1, /* a bounded cross-workgroup wait of the step kernel ran out          */
+  LR_DEV_POS_RANGE = 2     /* a position outside the KV cache or the RoPE table                  */
+};
+
 /* Library version (major*10000 + minor*100 + patch) and text for an LR_E_* code. */
 int lr_version(void);
 const char* lr_error_string(int code);
@@ -69,11 +77,24 @@ int lr_add_rmsnorm(const void* resid_in, const void* d1, const void* d2, const v
 /* y[m, n] = bf16( sum_k x[m, k] * w[n, k] )   x [M, K] (row stride ldx), w [N, K] dense,
  * y [M, N] (row stride ldy).  nn.Linear without bias: wqkv / wo (utils.py:191, 258), w1 / w2
  * (utils.py:146, 148), wqkv1 (utils.py:311), output (gpt_ladder_TP.py:283).
- * M <= 8 runs the weight-streaming GEMV, larger M the LDS-tiled MFMA GEMM.  K % 8 == 0.
+ * K % 8 == 0.  The kernel is chosen from the shape: M <= 4 (and M <= 8 with act_swiglu) the
+ * weight-streaming GEMV (v_dot2 on packed pairs, every weight read once); 4 < M <= 8 on a matrix
+ * with few rows two GEMV passes of four rows; 4 < M <= 64 the skinny matrix-core GEMM (32 weight
+ * rows per workgroup, K split over the waves); M >= 512 on a large enough grid the 256 x 256 tile
+ * matrix-core GEMM; everything else the 128 x 128 tile matrix-core GEMM.  All of them accumulate
+ * in fp32 and round once; the summation order, hence the last bit, depends on the kernel.
  * act_swiglu != 0: x is taken to be [M, 2K] = [u | g] (row stride ldx) and the kernel consumes
  * bf16( bf16(silu(g)) * u ) in its place -- w2(silu(g) * u), utils.py:147-148. */
 int lr_linear(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K, int act_swiglu,
               lr_stream_t stream);
+
+/* lr_linear with the launch configuration of the GEMV given by the caller instead of chosen from
+ * the shape: gemv_cfg = rows per wave * 100 + K-split * 10 + unroll, one of 144, 212, 222, 242, 244,
+ * 412, 422, 442 (anything else: 242; 0: the shape heuristic, i.e. lr_linear).  Only consulted where
+ * lr_linear would run the GEMV.  No counterpart in the reference: for callers that tune per shape.
+ * Results do not depend on it beyond the fp32 summation order. */
+int lr_linear_tuned(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
+                    int act_swiglu, int gemv_cfg, lr_stream_t stream);
 
 /* out[r, i] = bf16( bf16(silu(h[r, I + i])) * h[r, i] ),  h [rows, 2I] = [u | g] (row stride ldh).
  * F.silu(g) * u after chunk(2), utils.py:147-148 and :386. */
@@ -88,10 +109,14 @@ int lr_swiglu(const void* h, int64_t ldh, void* out, int rows, int I, lr_stream_
  * q is rotated IN PLACE; rotated k and raw v go to k_cache / v_cache [Bmax, Hkv, Smax, hd] at
  * slot pos[s] (apply_rotary_emb utils.py:120-132, 197-198; KVCache.update utils.py:50-59,
  * 248-250).  Rotation is done in fp32 on interleaved pairs with separately rounded products.
- * Rows whose position is outside [0, Smax) (or outside the table) are left untouched. */
+ * Rows whose position is outside [0, Smax) (or outside the table) are left untouched -- nothing is
+ * rotated, nothing is written to the cache -- and, if `err` is not NULL, the device word *err
+ * (int32) is set to LR_DEV_POS_RANGE.  The reference fails with an index error there
+ * (utils.py:55, gpt_ladder_TP.py:255); a device-side check cannot raise, so the caller reads the
+ * word when it next synchronises.  The word is only ever set, never cleared, by the library. */
 int lr_rope_kv_write(void* qkv, int64_t ldqkv, const void* table, int table_is_gathered, const int32_t* pos,
                      void* k_cache, void* v_cache, int B, int S, int Hq, int Hkv, int hd, int Smax, int block_size,
-                     lr_stream_t stream);
+                     int32_t* err, lr_stream_t stream);
 
 /* Bytes of fp32 scratch lr_attn_decode needs for (B, Hq, hd, Smax). */
 size_t lr_attn_decode_scratch_bytes(int B, int Hq, int hd, int Smax);
@@ -149,6 +174,8 @@ typedef struct {
 typedef struct {
   int32_t dim, n_layer, n_head, n_kv_head, head_dim, ffn, out_rows, vocab, smax, block_size;
   float eps;
+  int32_t attention_workgroups; /* 0: chosen by the library; > 0: use at least this many workgroups for
+                                   attention (fewer keys each, at most 16) -- part of the workspace layout */
   const void *tok_embeddings, *norm, *output, *freqs_cis; /* [vocab, dim], [dim], [out_rows, dim], table */
   const lr_layer_t* layers_dev;                           /* DEVICE array of n_layer entries            */
 } lr_ladder_model_t;
@@ -167,9 +194,15 @@ int lr_ladder_step_init(const lr_ladder_model_t* model, int batch, void* workspa
  * so that replaying the captured step is a complete decode loop.  tokens and cur_token may alias.
  * The kernel occupies every CU (one resident workgroup each) and the workgroups wait for each
  * other's results: nothing else may run on the device concurrently, and two steps must not
- * overlap.  Every wait is bounded; if one ever expires the workspace word at
- * lr_ladder_step_fail_offset() becomes non-zero, the outputs of that step are undefined and the
- * workspace must be initialised again. */
+ * overlap.  The workspace layout depends on the descriptor (smax, attention_workgroups, ...):
+ * size, initialise and step with the same descriptor values.
+ * Device-side failures: every wait is bounded, and if one ever expires the int32 workspace word at
+ * lr_ladder_step_fail_offset() becomes LR_DEV_WAIT_EXPIRED; a position pos[0] outside
+ * [0, min(smax, block_size)) makes it LR_DEV_POS_RANGE and the step computes and writes nothing
+ * (the per-op path treats such a position the same way, see lr_rope_kv_write).  Once the word is
+ * non-zero the outputs are undefined, later steps on that workspace return at once without
+ * computing, and the workspace must be initialised again: callers read the word whenever they
+ * synchronise anyway (after a generation, after a timed loop) and raise. */
 int lr_ladder_decode_step(const lr_ladder_model_t* model, int batch, const int32_t* tokens, int32_t* pos, void* logits,
                           int64_t ldl, int32_t* next_token, int advance, int32_t* cur_token, int32_t* history,
                           int64_t ld_hist, int hist_len, int pos0, void* workspace, size_t bytes, lr_stream_t stream);
@@ -183,21 +216,6 @@ size_t lr_ladder_step_fail_offset(void);
  * torch.empty_like(probs).exponential_(1), benchmark.py:59), `probs` is optional (bf16 [B][ldp]). */
 int lr_sample_topk(const void* logits, int64_t ldl, const void* noise, int64_t ldn, int B, int V, float temperature,
                    int top_k, void* probs, int64_t ldp, int32_t* next_token, lr_stream_t stream);
-
-/* Tuning hook, no counterpart in the reference: use at least this many attention workgroups in
- * the step kernel (more workgroups, fewer keys each; <= 0 restores the default).  Set it before the
- * workspace is sized and initialised. */
-void lr_ladder_step_tune(int attention_workgroups);
-
-/* Debug hook, no counterpart in the reference: following steps record, per workgroup, up to 12 wall-clock
- * stamps (100 MHz) for 4 consecutive slots starting at `first_slot` into `device_buffer` (NULL
- * switches it off).  Returns the bytes the buffer must hold. */
-size_t lr_ladder_step_profile(void* device_buffer, int first_slot);
-
-/* Tuning hook, no counterpart in the reference: force the GEMV launch configuration
- * (rows-per-wave * 100 + K-split * 10 + unroll; 0 restores the built-in shape heuristic).
- * Results do not depend on it beyond fp32 summation order. */
-void lr_gemv_set_cfg(int cfg);
 
 #ifdef __cplusplus
 }

@@ -139,10 +139,19 @@ def generate(model, prompt: torch.Tensor, max_new_tokens: int, batch_size: int, 
                                    callback=callback, **sampling_kwargs)
     device_sync(device)
     decode_latency = time.perf_counter() - t0
+    _raise_on_device_error(model)
     print_rank_0(f"Decode latency: {decode_latency} sec")
     if generated:
         empty[:, T + 1:] = torch.cat(generated, dim=-1)
     return empty, decode_latency, prefill_latency
+
+
+def _raise_on_device_error(model):
+    """After a synchronisation: a latency measured over steps that did no work (a position beyond the
+    cache, an expired wait in the one-kernel step) must never be reported as a result."""
+    check = getattr(model, "check_device_errors", None)
+    if check is not None:
+        check()
 
 
 class DecodeGraph:
@@ -231,6 +240,7 @@ def generate_using_cuda_graphs(prefill_graph, static_x, static_input_pos, static
         decode_graph.replay()
     device_sync(device)
     decode_latency = time.perf_counter() - t0
+    _raise_on_device_error(decode_graph.model)
     print_rank_0(f"Decode latency: {decode_latency} sec")
     if num_new_tokens > 1:
         empty[:, T + 1:] = decode_graph.history[:, : num_new_tokens - 1]
@@ -363,6 +373,7 @@ def main(model_name: str, prompt_length: int = 1, num_samples: int = 5, max_new_
                     decode_graph.replay()
                 device_sync(device)
                 decode_latency = time.perf_counter() - t1
+                _raise_on_device_error(model)
                 print_rank_0(f"Decode latency: {decode_latency} sec")
                 if max_new_tokens > 1:
                     empty[:, T + 1:] = decode_graph.history[:, : max_new_tokens - 1]

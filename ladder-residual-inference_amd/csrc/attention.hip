@@ -7,9 +7,12 @@
 // Only slots <= pos are touched: with the reference's boolean mask the other slots get weight
 // exp(-inf) = 0, so this is the same function of the cache.
 //
-// Prefill (S queries per sequence): one lane per query row with the running (max, sum, output)
-// in registers, K/V tiles of 32 keys broadcast from LDS as fp32.  Exact fp32 softmax, one rounding
-// at the end.
+// Prefill (S >= 16 queries per sequence): flash-style causal attention on the matrix cores in the
+// transposed form (k_attn_prefill_mfma below: a query is a lane, four waves share K / V^T tiles in
+// LDS, P enters the second product as bf16 hi + lo so the fp32 softmax weights survive).  Shorter
+// inputs (1 < S < 16) use the older lane-per-query kernel (k_attn_prefill: running max / sum /
+// output in registers, K/V tiles of 32 keys broadcast from LDS as fp32).  Both: exact fp32
+// softmax semantics, one rounding of the output.
 #include "lr_common.h"
 
 // ------------------------------------------------------------------------------------ decode

@@ -200,12 +200,15 @@ __global__ __launch_bounds__(256) void k_rope_kv_write(u16* qkv, int64_t ldqkv, 
                                                        int table_is_gathered, const int32_t* __restrict__ pos,
                                                        u16* __restrict__ k_cache,
                                                        u16* __restrict__ v_cache, int S, int Hq, int Hkv, int hd,
-                                                       int Smax, int block_size) {
+                                                       int Smax, int block_size, int32_t* err) {
   const int row = blockIdx.x;  // b * S + s
   const int b = row / S, s = row - b * S;
   const int p = pos[s];
   const int trow_idx = table_is_gathered ? s : p;
-  if (p < 0 || p >= Smax || trow_idx >= block_size) return;
+  if (p < 0 || p >= Smax || trow_idx >= block_size) {
+    if (err && threadIdx.x == 0) *err = LR_DEV_POS_RANGE;
+    return;
+  }
   const int nq = Hq * hd, nkv = Hkv * hd;
   u16* x = qkv + (int64_t)row * ldqkv;
   const u16* trow = table + (int64_t)trow_idx * hd;
@@ -225,7 +228,7 @@ __global__ __launch_bounds__(256) void k_rope_kv_write(u16* qkv, int64_t ldqkv, 
 
 extern "C" int lr_rope_kv_write(void* qkv, int64_t ldqkv, const void* table, int table_is_gathered,
                                 const int32_t* pos, void* k_cache, void* v_cache, int B, int S, int Hq, int Hkv,
-                                int hd, int Smax, int block_size, lr_stream_t stream) {
+                                int hd, int Smax, int block_size, int32_t* err, lr_stream_t stream) {
   LR_REQUIRE_PTR(qkv);
   LR_REQUIRE_PTR(table);
   LR_REQUIRE_PTR(k_cache);
@@ -236,7 +239,7 @@ extern "C" int lr_rope_kv_write(void* qkv, int64_t ldqkv, const void* table, int
   if (hd % 8 || ldqkv % 8) return LR_E_ALIGN;
   k_rope_kv_write<<<dim3(B * S), dim3(256), 0, (hipStream_t)stream>>>((u16*)qkv, ldqkv, (const u16*)table,
                                                                       table_is_gathered, pos, (u16*)k_cache,
-                                                                      (u16*)v_cache, S, Hq, Hkv, hd, Smax, block_size);
+                                                                      (u16*)v_cache, S, Hq, Hkv, hd, Smax, block_size, err);
   return lr_launch_status();
 }
 

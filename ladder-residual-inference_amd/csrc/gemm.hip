@@ -11,7 +11,7 @@
 #include <type_traits>
 
 int lr_gemv_dispatch(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
-                     int act_swiglu, hipStream_t s);
+                     int act_swiglu, int gemv_cfg, hipStream_t s);
 
 constexpr int BM = 128, BN = 128, BK = 64, LDT = BK + 8;  // LDT: padded LDS row length in elements
 
@@ -435,8 +435,8 @@ __global__ __launch_bounds__(SW * 64) void k_gemm_skinny(const u16* __restrict__
   }
 }
 
-extern "C" int lr_linear(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
-                         int act_swiglu, lr_stream_t stream) {
+extern "C" int lr_linear_tuned(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
+                               int act_swiglu, int gemv_cfg, lr_stream_t stream) {
   LR_REQUIRE_PTR(x);
   LR_REQUIRE_PTR(w);
   LR_REQUIRE_PTR(y);
@@ -444,14 +444,14 @@ extern "C" int lr_linear(const void* x, int64_t ldx, const void* w, void* y, int
   if (ldx < (act_swiglu ? 2 : 1) * (int64_t)K || ldy < N) return LR_E_SHAPE;
   if (K % 8 || ldx % 8) return LR_E_ALIGN;
   hipStream_t s = (hipStream_t)stream;
-  if (M <= 4 || (act_swiglu && M <= 8)) return lr_gemv_dispatch(x, ldx, w, y, ldy, M, N, K, act_swiglu, s);
+  if (M <= 4 || (act_swiglu && M <= 8)) return lr_gemv_dispatch(x, ldx, w, y, ldy, M, N, K, act_swiglu, gemv_cfg, s);
   if (!act_swiglu && M <= 8 && (N + SN - 1) / SN < 96) {
     // few weight rows (the wqkv of a rank shard): 32-row workgroups would leave most CUs idle, so the
     // GEMV kernel (a row per wave, every CU busy) runs twice, four input rows each; the second pass
     // finds the weights in the memory-side cache
-    const int rc = lr_gemv_dispatch(x, ldx, w, y, ldy, 4, N, K, 0, s);
+    const int rc = lr_gemv_dispatch(x, ldx, w, y, ldy, 4, N, K, 0, 0, s);
     if (rc != LR_OK) return rc;
-    return lr_gemv_dispatch((const u16*)x + 4 * ldx, ldx, w, (u16*)y + 4 * ldy, ldy, M - 4, N, K, 0, s);
+    return lr_gemv_dispatch((const u16*)x + 4 * ldx, ldx, w, (u16*)y + 4 * ldy, ldy, M - 4, N, K, 0, 0, s);
   }
   if (!act_swiglu && M <= 64 && ldy % 2 == 0 && (int64_t)64 * ldx * 2 < 0x7fffffff && (int64_t)SN * K * 2 < 0x7fffffff) {
     const dim3 sgrid((N + SN - 1) / SN);
@@ -471,4 +471,9 @@ extern "C" int lr_linear(const void* x, int64_t ldx, const void* w, void* y, int
   else
     k_gemm<false><<<grid, dim3(256), 0, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy, M, N, K);
   return lr_launch_status();
+}
+
+extern "C" int lr_linear(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
+                         int act_swiglu, lr_stream_t stream) {
+  return lr_linear_tuned(x, ldx, w, y, ldy, M, N, K, act_swiglu, 0, stream);
 }

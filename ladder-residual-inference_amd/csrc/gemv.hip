@@ -171,13 +171,10 @@ static int pick_cfg(int M, int N, int K) {
   return R * 100 + ksplit * 10 + U;
 }
 
-int lr_gemv_override_cfg = 0;  // test / tuning hook: non-zero forces a configuration
-
-extern "C" void lr_gemv_set_cfg(int cfg) { lr_gemv_override_cfg = cfg; }
-
+// gemv_cfg: rows-per-wave * 100 + K-split * 10 + unroll, or 0 for the shape heuristic
 int lr_gemv_dispatch(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
-                     int act_swiglu, hipStream_t s) {
-  const int cfg = lr_gemv_override_cfg ? lr_gemv_override_cfg : pick_cfg(M, N, K);
+                     int act_swiglu, int gemv_cfg, hipStream_t s) {
+  const int cfg = gemv_cfg ? gemv_cfg : pick_cfg(M, N, K);
   const u16* xp = (const u16*)x;
   const u16* wp = (const u16*)w;
   u16* yp = (u16*)y;

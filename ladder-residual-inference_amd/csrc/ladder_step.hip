@@ -85,9 +85,10 @@ constexpr int POLL_SLEEP = 2;
 
 struct Ctrl {
   unsigned epoch_base, _p0[31];  // slots consumed by earlier steps (tags continue from here)
-  unsigned fail, _p1[31];
+  unsigned fail, _p1[31];  // 0 = healthy; FAIL_WAIT: a bounded wait expired; FAIL_POS: position outside the cache / RoPE table
   unsigned nwg, _p2[31];
 };
+constexpr unsigned FAIL_WAIT = 1u, FAIL_POS = 2u;
 
 struct LayerPtrs {
   const u16 *wqkv, *wo, *w1, *w2, *attn_norm, *ffn_norm;
@@ -178,9 +179,12 @@ struct Coh {
     __builtin_amdgcn_raw_buffer_store_b64(w, r, wo * 4, 0, AUX_SC1);
   }
   __device__ __forceinline__ bool give_up(unsigned& spins) const {
-    if ((++spins & 255u) == 0 && (spins > SPIN_LIMIT || cldu(fail))) {
-      cstu(fail, 1u);
-      return true;
+    if ((++spins & 255u) == 0) {
+      const unsigned f = cldu(fail);
+      if (spins > SPIN_LIMIT || f) {
+        if (f == 0) cstu(fail, FAIL_WAIT);
+        return true;
+      }
     }
     return false;
   }
@@ -1173,7 +1177,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   float* vnew = knew + HD;                              // [HD]
   float* s_m = vnew + HD;                               // [G]
   float* s_l = s_m + G;                                 // [G]
-  float* wbuf = s_l + G;                                // [M * Hq][NA_MAX]
+  float* wbuf = s_m + ((2 * G + 3) & ~3);               // [M * Hq][NA_MAX]   (what follows stays 16-byte aligned for odd G)
   float* cand_v = wbuf + M * Hq * NA_MAX;               // [NJMAX * M]
   int* cand_i = reinterpret_cast<int*>(cand_v + NJMAX * M);
   int* s_flag = cand_i + NJMAX * M;                     // [8]
@@ -1187,15 +1191,25 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   Coh coh;
   coh.r = __builtin_amdgcn_make_buffer_rsrc(p.ws, 0, (int)p.ws_bytes, 0x00020000);
   coh.fail = &ctrl->fail;
-  if (tid == 0) s_flag[1] = (int)cldu(&ctrl->epoch_base);
+  if (tid == 0) {
+    s_flag[1] = (int)cldu(&ctrl->epoch_base);
+    s_flag[0] = (int)cldu(&ctrl->fail);
+  }
   build_job_table(p, jtab, Hq * HD, w, nwg);
   if (tid < 32 && (tid >> 4) < L) lring[tid] = reinterpret_cast<const u32*>(p.layers)[tid];  // layers 0 and 1
   wg_sync();
   build_row_table(jtab, jtab + JK_COUNT * NW * 16);
   wg_sync();
   const unsigned epoch_base = (unsigned)s_flag[1];
-  int pos = p.pos[0];
-  pos = pos < 0 ? 0 : (pos >= p.Smax ? p.Smax - 1 : pos);
+  const int pos = p.pos[0];
+  // A position outside the cache or the RoPE table: nothing is computed or written (every workgroup
+  // takes the same decision from the same word), the failure word says why.  A workspace whose
+  // failure word is already set stays out of service until it is initialised again.
+  if (pos < 0 || pos >= p.Smax || pos >= p.block_size) {
+    if (w == 0 && tid == 0 && s_flag[0] == 0) cstu(&ctrl->fail, FAIL_POS);
+    return;
+  }
+  if (s_flag[0]) return;
   const bool att_wg = w < NA;
   // attention key range of this workgroup
   const int nkeys = pos + 1;
@@ -1370,12 +1384,17 @@ static int num_cus() {
   return n;
 }
 
-// keys one attention workgroup can hold in registers
-static int att_capacity(int hd) { return ATT_NI * NW * (64 / (hd / 8)); }
+// keys one attention workgroup can hold in registers: the V groups (ATT_NI * NW * keys per wave)
+// and the K tiles of the score pass (ATT_KT * NW * 32) both have to cover its key range
+static int att_capacity(int hd) {
+  const int v_keys = ATT_NI * NW * (64 / (hd / 8)), k_keys = ATT_KT * NW * 32;
+  return v_keys < k_keys ? v_keys : k_keys;
+}
+// LDS row length of the score buffer (the larger of the two, so either bound may be the binding one)
+static int att_sc_ld(int hd) { return ATT_NI * NW * (64 / (hd / 8)); }
 
-int g_na_override = -1;  // tuning hook: number of attention workgroups (must still cover Smax)
-
-static int pick_na(int Smax, int hd, int nwg) {
+// `want_na` > 0: the caller's lower bound for the number of attention workgroups (lr_ladder_model_t)
+static int pick_na(int Smax, int hd, int nwg, int want_na) {
   const int cap = att_capacity(hd);
   int na = (Smax + cap - 1) / cap;
   // more attention workgroups than capacity requires pay off up to about 128 keys each: attention is
@@ -1384,7 +1403,8 @@ static int pick_na(int Smax, int hd, int nwg) {
   if (want > NA_MAX) want = NA_MAX;
   if (want > nwg / 8) want = nwg / 8;
   if (want > na) na = want;
-  if (g_na_override > 0) na = g_na_override > na ? g_na_override : na;
+  if (want_na > NA_MAX) want_na = NA_MAX;
+  if (want_na > na) na = want_na;
   if (na < 1) na = 1;
   if (na >= nwg) na = nwg - 1;
   return na;
@@ -1393,7 +1413,7 @@ static int pick_na(int Smax, int hd, int nwg) {
 static Layout make_layout(const lr_ladder_model_t* md, int B, int nwg) {
   const int D = md->dim, Hq = md->n_head, hd = md->head_dim;
   const int nqkv = (Hq + 2 * md->n_kv_head) * hd;
-  const int na = pick_na(md->smax, hd, nwg);
+  const int na = pick_na(md->smax, hd, nwg, md->attention_workgroups);
   auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
   Layout l;
   size_t o = 0;
@@ -1426,8 +1446,8 @@ static bool has_instance(int B, int hd, int G) {
 template <int M, int HD, int G>
 static size_t lds_bytes(int D, int I, int Hq) {
   const int xlen = M * (D > I ? D : I);
-  const size_t fl = (size_t)NW * NJMAX * M + NW * M * 2 + G * HD + (size_t)G * att_capacity(HD) + NW * G * HD +
-                    2 * HD + 2 * G + (size_t)M * Hq * NA_MAX + 2 * NJMAX * M + 8 + 64 + JK_COUNT * NW * 16 + JK_COUNT * NJMAX;
+  const size_t fl = (size_t)NW * NJMAX * M + NW * M * 2 + G * HD + (size_t)G * att_sc_ld(HD) + NW * G * HD +
+                    2 * HD + ((2 * G + 3) & ~3) + (size_t)M * Hq * NA_MAX + 2 * NJMAX * M + 8 + 64 + JK_COUNT * NW * 16 + JK_COUNT * NJMAX;
   return ((size_t)xlen * 2 + (size_t)M * D) * sizeof(u16) + fl * sizeof(float) + 16;
 }
 
@@ -1443,6 +1463,8 @@ static int validate(const lr_ladder_model_t* md, int B) {
   if (B < 1 || md->dim <= 0 || md->n_layer <= 0 || md->n_head <= 0 || md->n_kv_head <= 0 || md->ffn <= 0 ||
       md->out_rows <= 0 || md->vocab <= 0 || md->smax <= 0 || md->block_size <= 0 || md->n_head % md->n_kv_head)
     return LR_E_SHAPE;
+  // every cache slot needs a row of the RoPE table (block_size rows); the cache length itself is rounded up to 8
+  if (md->smax > ((md->block_size + 7) & ~7)) return LR_E_SHAPE;
   if (B > 2 || md->dim > PRO_NIT * NT * 8 || md->dim % 8 || md->ffn % 8 || (md->head_dim != 64 && md->head_dim != 128))
     return LR_E_UNSUPPORTED;
   const int G = md->n_head / md->n_kv_head;
@@ -1451,7 +1473,7 @@ static int validate(const lr_ladder_model_t* md, int B) {
   if (lds_need(B, md->head_dim, G, md->dim, md->ffn, md->n_head) > 160 * 1024) return LR_E_UNSUPPORTED;
   const int nwg = num_cus();
   if (nwg < 2) return LR_E_LAUNCH;
-  const int na = pick_na(md->smax, md->head_dim, nwg);
+  const int na = pick_na(md->smax, md->head_dim, nwg, md->attention_workgroups);
   if (na > NA_MAX || (md->smax + na - 1) / na > att_capacity(md->head_dim)) return LR_E_UNSUPPORTED;
   if (!md->tok_embeddings || !md->norm || !md->output || !md->freqs_cis || !md->layers_dev) return LR_E_NULL;
   return LR_OK;
@@ -1471,18 +1493,23 @@ static int launch_step(const StepParams& sp, int Hq, hipStream_t s) {
   return lr_launch_status();
 }
 
-unsigned long long* g_prof = nullptr;  // debug hook: device buffer for phase timestamps
+#ifdef LR_STEP_PROFILE
+unsigned long long* g_prof = nullptr;  // device buffer for phase timestamps
 int g_prof_t0 = 0;
+#endif
 
 }  // namespace
 
-extern "C" void lr_ladder_step_tune(int attention_workgroups) { g_na_override = attention_workgroups; }
-
+#ifdef LR_STEP_PROFILE
+// Debug builds only (not declared in the public header): following steps record, per workgroup,
+// wall-clock stamps (100 MHz) for PROF_SLOTS consecutive slots starting at `first_slot` into
+// `device_buffer` (NULL switches it off).  Returns the bytes the buffer must hold.
 extern "C" size_t lr_ladder_step_profile(void* device_buffer, int first_slot) {
   g_prof = reinterpret_cast<unsigned long long*>(device_buffer);
   g_prof_t0 = first_slot;
   return (size_t)num_cus() * PROF_SLOTS * PROF_POINTS * sizeof(unsigned long long);
 }
+#endif
 
 extern "C" size_t lr_ladder_step_workspace_bytes(const lr_ladder_model_t* md, int batch) {
   if (validate(md, batch) != LR_OK) return 0;
@@ -1522,7 +1549,7 @@ extern "C" int lr_ladder_decode_step(const lr_ladder_model_t* md, int batch, con
   StepParams sp;
   sp.D = md->dim; sp.L = md->n_layer; sp.Hkv = md->n_kv_head; sp.I = md->ffn; sp.V = md->out_rows;
   sp.vocab = md->vocab; sp.Smax = md->smax; sp.block_size = md->block_size; sp.B = batch;
-  sp.NA = pick_na(md->smax, md->head_dim, nwg);
+  sp.NA = pick_na(md->smax, md->head_dim, nwg, md->attention_workgroups);
   sp.nqkv = (md->n_head + 2 * md->n_kv_head) * md->head_dim;
   sp.eps = md->eps;
   sp.tok_emb = (const u16*)md->tok_embeddings; sp.final_norm = (const u16*)md->norm;
@@ -1537,8 +1564,13 @@ extern "C" int lr_ladder_decode_step(const lr_ladder_model_t* md, int batch, con
   sp.oqkv = (unsigned)(l.qkv / 4); sp.oact = (unsigned)(l.act / 4);
   sp.oopart = (unsigned)(l.opart / 4); sp.omlpart = (unsigned)(l.mlpart / 4); sp.ocand = (unsigned)(l.cand / 4);
   sp.odone = (unsigned)(l.done / 4); sp.oy = (unsigned)(l.y / 4);
+#ifdef LR_STEP_PROFILE
   sp.prof = g_prof;
   sp.prof_t0 = g_prof_t0;
+#else
+  sp.prof = nullptr;
+  sp.prof_t0 = 0;
+#endif
   hipStream_t s = (hipStream_t)stream;
   const int G = md->n_head / md->n_kv_head, hd = md->head_dim;
 #define LR_STEP(MV, HDV, GV) \

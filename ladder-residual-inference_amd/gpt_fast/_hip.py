@@ -21,9 +21,11 @@ _PROTOS = {
     "lr_add_rmsnorm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float,
                                c_void_p]),
     "lr_linear": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
+    "lr_linear_tuned": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int,
+                                c_void_p]),
     "lr_swiglu": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_int, c_void_p]),
     "lr_rope_kv_write": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                                 c_int, c_int, c_int, c_int, c_void_p]),
+                                 c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "lr_attn_decode_scratch_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "lr_attn_decode": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int,
                                c_int, c_int, c_void_p, c_size_t, c_void_p]),
@@ -34,21 +36,18 @@ _PROTOS = {
     "lr_sample_topk": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_float, c_int, c_void_p, c_int64,
                                c_void_p, c_void_p]),
     "lr_advance": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_void_p]),
-    "lr_gemv_set_cfg": (None, [c_int]),
     "lr_ladder_step_workspace_bytes": (c_size_t, [c_void_p, c_int]),
     "lr_ladder_step_init": (c_int, [c_void_p, c_int, c_void_p, c_size_t, c_void_p]),
     "lr_ladder_decode_step": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_void_p,
                                       c_void_p, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "lr_ladder_step_fail_offset": (c_size_t, []),
-    "lr_ladder_step_tune": (None, [c_int]),
-    "lr_ladder_step_profile": (c_size_t, [c_void_p, c_int]),
 }
 
 
 class LadderModelDesc(ctypes.Structure):
     """lr_ladder_model_t of include/ladder_hip.h (per-rank sizes)."""
     _fields_ = [(n, c_int32) for n in ("dim", "n_layer", "n_head", "n_kv_head", "head_dim", "ffn", "out_rows", "vocab",
-                                       "smax", "block_size")] + [("eps", c_float)] + \
+                                       "smax", "block_size")] + [("eps", c_float), ("attention_workgroups", c_int32)] + \
                [(n, c_void_p) for n in ("tok_embeddings", "norm", "output", "freqs_cis", "layers_dev")]
 
 
@@ -142,14 +141,20 @@ def add_rmsnorm(resid_in, d1, d2, gain, resid_out, normed_out, eps: float):
     return normed_out
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, act_swiglu: bool = False):
-    """out[M, N] = x[M, K] @ w[N, K]^T (x = [u | g] of width 2K when act_swiglu)."""
+def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, act_swiglu: bool = False, gemv_cfg: int = 0):
+    """out[M, N] = x[M, K] @ w[N, K]^T (x = [u | g] of width 2K when act_swiglu).  gemv_cfg != 0 goes
+    through lr_linear_tuned (an explicit GEMV launch configuration for this one call)."""
     M, xc, ldx = _rows_ld(x)
     N, K = w.shape
     assert w.is_contiguous() and xc == (2 * K if act_swiglu else K), (x.shape, w.shape, act_swiglu)
     Mo, No, ldy = _rows_ld(out)
     assert (Mo, No) == (M, N), (out.shape, M, N)
-    _check(load().lr_linear(_dev(x), ldx, _dev(w), _dev(out), ldy, M, N, K, int(act_swiglu), _stream()), "lr_linear")
+    if gemv_cfg:
+        _check(load().lr_linear_tuned(_dev(x), ldx, _dev(w), _dev(out), ldy, M, N, K, int(act_swiglu), int(gemv_cfg),
+                                      _stream()), "lr_linear_tuned")
+    else:
+        _check(load().lr_linear(_dev(x), ldx, _dev(w), _dev(out), ldy, M, N, K, int(act_swiglu), _stream()),
+               "lr_linear")
     return out
 
 
@@ -173,6 +178,42 @@ def swiglu(h: torch.Tensor, out: torch.Tensor):
     return out
 
 
+def device_error_word(device) -> torch.Tensor:
+    """One int32 word per device that kernels set (never clear) when they meet a condition only the
+    device can see -- a position outside the KV cache or the RoPE table.  Read by
+    raise_on_device_error() at the caller's next synchronisation point."""
+    key = torch.device(device)
+    if key.index is None:
+        key = torch.device("cuda", torch.cuda.current_device())
+    w = _ERR_WORDS.get(key)
+    if w is None:
+        w = _ERR_WORDS[key] = torch.zeros(1, dtype=torch.int32, device=key)
+    return w
+
+
+_ERR_WORDS = {}
+DEV_WAIT_EXPIRED, DEV_POS_RANGE = 1, 2
+_DEV_ERR_TEXT = {DEV_WAIT_EXPIRED: "a bounded cross-workgroup wait of the decode-step kernel expired",
+                 DEV_POS_RANGE: "a position outside the KV cache or the RoPE table was used"}
+
+
+def raise_on_device_error(device=None, fused_steps=()):
+    """Synchronising check of the device-side error words: the per-device word of the per-op kernels
+    and the failure word of every FusedLadderStep given.  Raises LadderHipError and clears the
+    per-device word (a failed step workspace must be reset by its owner)."""
+    words = list(_ERR_WORDS.items()) if device is None else [(torch.device(device), device_error_word(device))]
+    for dev, w in words:
+        code = int(w.item())
+        if code:
+            w.zero_()
+            raise LadderHipError(f"device-side error on {dev}: {_DEV_ERR_TEXT.get(code, code)}")
+    for fs in fused_steps:
+        code = fs.fail_code() if fs is not None else 0
+        if code:
+            raise LadderHipError(f"decode-step kernel failed: {_DEV_ERR_TEXT.get(code, code)}; "
+                                 "its workspace has to be initialised again (FusedLadderStep.reset)")
+
+
 def rope_kv_write(qkv, table, table_is_gathered, pos, k_cache, v_cache, B, S, Hq, Hkv, hd):
     rows, cols, ld = _rows_ld(qkv)
     assert rows == B * S and pos.dtype == torch.int32 and pos.is_cuda and pos.numel() == S
@@ -180,7 +221,8 @@ def rope_kv_write(qkv, table, table_is_gathered, pos, k_cache, v_cache, B, S, Hq
     Bmax, hkv_c, Smax, hd_c = k_cache.shape
     assert B <= Bmax and hkv_c == Hkv and hd_c == hd and table.is_contiguous() and table.shape[-2:] == (hd // 2, 2)
     _check(load().lr_rope_kv_write(_dev(qkv), ld, _dev(table), int(bool(table_is_gathered)), pos.data_ptr(),
-                                   _dev(k_cache), _dev(v_cache), B, S, Hq, Hkv, hd, Smax, table.shape[0], _stream()),
+                                   _dev(k_cache), _dev(v_cache), B, S, Hq, Hkv, hd, Smax, table.shape[0],
+                                   device_error_word(qkv.device).data_ptr(), _stream()),
            "lr_rope_kv_write")
 
 
@@ -253,7 +295,7 @@ class FusedLadderStep:
     table, the model descriptor and the (initialised) workspace.  Keeps references to every tensor
     whose address it handed to the library."""
 
-    def __init__(self, model, batch: int):
+    def __init__(self, model, batch: int, attention_workgroups: int = 0):
         cfg = model.config
         dev = model.output.weight.device
         rows = []
@@ -271,7 +313,8 @@ class FusedLadderStep:
         self.desc = LadderModelDesc(
             dim=cfg.dim, n_layer=cfg.n_layer, n_head=cfg.n_head_local, n_kv_head=cfg.n_kv_local, head_dim=cfg.head_dim,
             ffn=cfg.ffn_local, out_rows=cfg.output_rows, vocab=cfg.vocab_size, smax=model.max_seq_length,
-            block_size=cfg.block_size, eps=cfg.norm_eps, tok_embeddings=model.tok_embeddings.weight.data_ptr(),
+            block_size=cfg.block_size, eps=cfg.norm_eps, attention_workgroups=attention_workgroups,
+            tok_embeddings=model.tok_embeddings.weight.data_ptr(),
             norm=model.norm.weight.data_ptr(), output=model.output.weight.data_ptr(),
             freqs_cis=model.freqs_cis.data_ptr(), layers_dev=self.layer_table.data_ptr())
         self.batch = batch
@@ -289,10 +332,13 @@ class FusedLadderStep:
         _check(load().lr_ladder_step_init(ctypes.byref(self.desc), self.batch, self.workspace.data_ptr(), self.bytes,
                                           _stream()), "lr_ladder_step_init")
 
-    def failed(self) -> bool:
-        """Synchronises.  True if a barrier wait of an earlier step expired."""
+    def fail_code(self) -> int:
+        """Synchronises.  0, or the LR_DEV_* value an earlier step left in the workspace's failure word."""
         off = int(load().lr_ladder_step_fail_offset())
-        return bool(self.workspace[off:off + 4].view(torch.int32).item())
+        return int(self.workspace[off:off + 4].view(torch.int32).item())
+
+    def failed(self) -> bool:
+        return self.fail_code() != 0
 
     def step(self, tokens, pos, logits, next_token=None, advance=False, cur_token=None, history=None, pos0=0):
         B = self.batch

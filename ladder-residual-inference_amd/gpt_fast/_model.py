@@ -85,6 +85,10 @@ class GPTBase(nn.Module):
         cfg = self.config
         if cfg.head_dim not in (64, 128):
             raise NotImplementedError(f"head_dim {cfg.head_dim}: the attention kernels are built for 64 and 128")
+        if max_seq_length > cfg.block_size:
+            # the RoPE table has block_size rows: the reference fails with an index error at the first position
+            # beyond it (gpt_ladder_TP.py:255); here the mistake is reported before anything is allocated
+            raise ValueError(f"max_seq_length {max_seq_length} exceeds the model's block_size {cfg.block_size}")
         max_seq_length = find_multiple(max_seq_length, 8)
         self.max_seq_length = max_seq_length
         self.max_batch_size = max_batch_size
@@ -99,6 +103,15 @@ class GPTBase(nn.Module):
         # kept for API compatibility (the kernels derive visibility from input_pos)
         self.causal_mask = torch.tril(torch.ones(max_seq_length, max_seq_length, dtype=torch.bool, device=device))
         self._ws.clear()
+        _hip.device_error_word(device)  # exists before any step is captured into a graph
+
+    def check_device_errors(self):
+        """Synchronises, then raises LadderHipError if a kernel of an earlier call reported a condition
+        only the device can see: a position outside the KV cache / RoPE table (the reference raises
+        an index error there), or an expired wait inside the one-kernel decode step.  benchmark.py
+        calls it after every generation, next to the synchronisation it does anyway."""
+        fused = [f for f in getattr(self, "_fused", {}).values() if f is not None]
+        _hip.raise_on_device_error(self.output.weight.device, fused)
 
     def release_workspace(self):
         self._ws.clear()

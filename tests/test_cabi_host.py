@@ -141,3 +141,57 @@ def test_bytes_per_step_accounting():
     assert bm.decode_bytes_per_step(c, 1, 2049) - b0 == 80 * 2 * 128 * 2
     # a second sequence adds its KV, embedding row and logits, not the weights
     assert bm.decode_bytes_per_step(c, 2, 2048) - b0 < 0.1e9
+
+
+def _desc(**over):
+    from gpt_fast import _hip
+
+    kw = dict(dim=256, n_layer=2, n_head=4, n_kv_head=2, head_dim=64, ffn=512, out_rows=512, vocab=512, smax=64,
+              block_size=64, eps=1e-5, attention_workgroups=0, tok_embeddings=4096, norm=4096, output=4096,
+              freqs_cis=4096, layers_dev=4096)
+    kw.update(over)
+    return _hip.LadderModelDesc(**kw)
+
+
+def test_step_descriptor_is_validated_on_the_host(lib):
+    """Shapes the one-kernel step must refuse are refused before any device is looked at (no GPU here)."""
+    import ctypes
+
+    E_NULL, E_SHAPE, E_UNSUPPORTED = -1, -3, -4
+    init = lambda d, b=1: lib.lr_ladder_step_init(ctypes.byref(d), b, 256, 1 << 20, None)
+    # a cache longer than the RoPE table: positions beyond block_size would read past the end of freqs_cis
+    assert init(_desc(smax=72, block_size=64)) == E_SHAPE
+    assert lib.lr_ladder_step_workspace_bytes(ctypes.byref(_desc(smax=72, block_size=64)), 1) == 0
+    assert init(_desc(smax=64, block_size=60)) != E_SHAPE          # the cache length is rounded up to 8
+    assert init(_desc(n_head=5)) == E_SHAPE                        # q heads not a multiple of kv heads
+    assert init(_desc(), b=3) == E_UNSUPPORTED                     # batch: 1 or 2
+    assert init(_desc(head_dim=48)) == E_UNSUPPORTED
+    assert init(_desc(dim=20000)) == E_UNSUPPORTED
+
+
+def test_load_hook_fuses_separate_projections():
+    """utils.py:178-185: checkpoints with wq / wk / wv load into the fused wqkv, rows [q; k; v]."""
+    from gpt_fast.config import ModelArgs
+    from gpt_fast.utils import Attention
+
+    cfg = ModelArgs(dim=64, n_head=4, n_local_heads=2, n_layer=1, intermediate_size=128)
+    att = Attention(cfg)
+    g = torch.Generator().manual_seed(0)
+    wq, wk, wv = (torch.randn(r, 64, generator=g) for r in (64, 32, 32))
+    wo = torch.randn(64, 64, generator=g)
+    att.load_state_dict({"wq.weight": wq, "wk.weight": wk, "wv.weight": wv, "wo.weight": wo})
+    assert torch.equal(att.wqkv.weight, torch.cat([wq, wk, wv])) and torch.equal(att.wo.weight, wo)
+    # an already fused checkpoint passes through untouched
+    att2 = Attention(cfg)
+    att2.load_state_dict(att.state_dict())
+    assert torch.equal(att2.wqkv.weight, att.wqkv.weight)
+
+
+def test_setup_caches_refuses_a_sequence_longer_than_block_size():
+    import benchmark as bm
+    from gpt_fast.config import ModelArgs
+
+    with torch.device("meta"):
+        model = bm.GPTLadder(ModelArgs(block_size=64, vocab_size=512, n_layer=1, n_head=4, dim=256))
+    with pytest.raises(ValueError):
+        model.setup_caches(1, 65)

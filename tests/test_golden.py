@@ -59,14 +59,12 @@ def test_fixtures_tell_the_schedules_apart():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("fused", [True, False])
-@pytest.mark.parametrize("family", FAMILIES)
+@pytest.mark.parametrize("family,fused", [("ladder", True)] + [(f, False) for f in FAMILIES])
 def test_hip_matches_fixture(family, fused):
+    """fused: the one-kernel decode step (it exists for the ladder schedule only)."""
     import benchmark as bm
     from gpt_fast.config import ModelArgs
 
-    if fused and family != "ladder":
-        pytest.skip("the one-kernel decode step exists for the ladder schedule only")
     P, prompt, tokens, logits, (B, T, NEW) = load(family)
     cls = {"ladder": bm.GPTLadder, "dense": bm.GPTDense, "desync": bm.GPTDesync, "parallel": bm.GPTParallel}[family]
     with torch.device("meta"):

@@ -134,8 +134,6 @@ GEMV_SHAPES = [  # (N, K): the 70B rank shard, the 8B model, the 1B model, and r
 @pytest.mark.parametrize("N,K", GEMV_SHAPES)
 @pytest.mark.parametrize("M", [1, 2, 3, 5, 8])
 def test_linear_gemv(hip, M, N, K):
-    if M in (2, 3, 5) and N * K > 20e6:
-        pytest.skip("odd batch sizes are covered on the smaller shapes")
     x = rnd(M, K, seed=8)
     w = rnd(N, K, seed=9, scale=0.02)
     y = torch.empty(M, N, dtype=BF, device=DEV)
@@ -151,8 +149,6 @@ def test_linear_gemv(hip, M, N, K):
 def test_linear_skinny_batches(hip, M, N, K):
     """Decode batches (4 < M <= 64) take the skinny matrix-core GEMM: ragged N, K not a multiple of the
     128-element tile, M on both sides of the 32-row column tile, a strided output view."""
-    if M in (31, 33) and N * K > 20e6:
-        pytest.skip("odd batch sizes are covered on the smaller shapes")
     x = rnd(M, K, seed=12)
     w = rnd(N, K, seed=13, scale=0.02)
     y = torch.empty(M, N, dtype=BF, device=DEV)
@@ -169,12 +165,7 @@ def test_linear_gemv_every_launch_configuration(hip, cfg):
     x = rnd(4, 3584, seed=10)
     w = rnd(1030, 3584, seed=11, scale=0.02)
     y = torch.empty(4, 1030, dtype=BF, device=DEV)
-    lib = hip.load()
-    try:
-        lib.lr_gemv_set_cfg(cfg)
-        hip.linear(x, w, y)
-    finally:
-        lib.lr_gemv_set_cfg(0)
+    hip.linear(x, w, y, gemv_cfg=cfg)   # lr_linear_tuned: the configuration is an argument of the call
     assert_close_ulp(y, linear_ref(x, w), what=f"gemv cfg {cfg}")
 
 
@@ -253,6 +244,29 @@ def test_rope_kv_write_exact(hip, hd, Hq, Hkv, gathered):
     assert torch.equal(work[..., : Hq * hd].reshape(B, S, Hq, hd), q_ref)
     assert torch.equal(kc, kc_ref) and torch.equal(vc, vc_ref)
     assert torch.equal(work[..., Hq * hd:], torch.cat([k, v], -1))   # k and v columns are left as they were
+
+
+def test_rope_kv_write_position_out_of_range_sets_the_error_word(hip):
+    """Positions beyond the cache or the RoPE table: the row is left alone, nothing lands in the cache and the
+    per-device error word becomes LR_DEV_POS_RANGE (the reference raises an index error, utils.py:55)."""
+    B, S, Smax, block, Hq, Hkv, hd = 1, 3, 16, 12, 2, 1, 64
+    qkv = rnd(B, S, (Hq + 2 * Hkv) * hd, seed=29)
+    before = qkv.clone()
+    table = O.rope_table(block, hd, 10000, BF).to(DEV)
+    kc = torch.zeros(B, Hkv, Smax, hd, dtype=BF, device=DEV)
+    vc = torch.zeros_like(kc)
+    word = hip.device_error_word(DEV)
+    word.zero_()
+    pos = torch.tensor([2, 16, 13], dtype=torch.int32, device=DEV)   # in range; beyond the cache; beyond the table
+    hip.rope_kv_write(qkv, table, False, pos, kc, vc, B, S, Hq, Hkv, hd)
+    torch.cuda.synchronize()
+    assert word.item() == hip.DEV_POS_RANGE
+    assert torch.equal(qkv[:, 1:], before[:, 1:]) and not torch.equal(qkv[:, 0], before[:, 0])
+    assert bool((kc[:, :, 3:] == 0).all()) and bool((kc[:, :, 2] != 0).any())
+    with pytest.raises(hip.LadderHipError):
+        hip.raise_on_device_error(DEV)
+    assert word.item() == 0      # reported once
+    hip.raise_on_device_error(DEV)
 
 
 # ------------------------------------------------------------------------------------ attention
