@@ -38,7 +38,8 @@ enum {
   LR_E_ALIGN = -2,       /* a pointer is not 16-byte aligned or a stride is not % 8      */
   LR_E_SHAPE = -3,       /* a size is non-positive or inconsistent                        */
   LR_E_UNSUPPORTED = -4, /* a size the kernels are not built for (e.g. head_dim)          */
-  LR_E_LAUNCH = -5       /* the HIP runtime refused the launch                            */
+  LR_E_LAUNCH = -5,      /* the HIP runtime refused the launch                            */
+  LR_E_TOO_LARGE = -6    /* more scratch needed than the library's built-in buffer holds  */
 };
 
 /* Values of device-side error words (lr_rope_kv_write's `err`, the workspace word at
@@ -131,6 +132,21 @@ size_t lr_attn_decode_scratch_bytes(int B, int Hq, int hd, int Smax);
 int lr_attn_decode(const void* q, int64_t ldq, const void* k_cache, const void* v_cache, const int32_t* pos, void* y,
                    int64_t ldy, int B, int Hq, int Hkv, int hd, int Smax, void* scratch, size_t scratch_bytes,
                    lr_stream_t stream);
+
+/* lr_attn_decode without a scratch argument, for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.
+ * The split-KV partial results go to a fixed device array inside the library
+ * (LR_ATTN_DECODE_STATIC_MAX_BYTES = 32 MiB, held by every GPU the library runs on until the
+ * process ends); the call allocates nothing and frees nothing.  Same kernels, same results as
+ * lr_attn_decode, bit for bit.  Limits: shapes whose lr_attn_decode_scratch_bytes() exceeds the
+ * array are refused with LR_E_TOO_LARGE (the 70B rank shard at batch 64 needs 17 MB); all calls on
+ * one GPU share the array, so calls that overlap on one GPU (two streams, two threads) race -- run
+ * them in stream order.  Nothing in the array has to start at a particular value: every word a
+ * call reads it has written itself.  The first call on a device looks up the array's address;
+ * make that call outside stream capture (a warm-up step does it). */
+#define LR_ATTN_DECODE_STATIC_MAX_BYTES ((size_t)32 << 20)
+int lr_attn_decode_static(const void* q, int64_t ldq, const void* k_cache, const void* v_cache, const int32_t* pos,
+                          void* y, int64_t ldy, int B, int Hq, int Hkv, int hd, int Smax, lr_stream_t stream);
 
 /* Causal attention of S query tokens per sequence against the cache (prefill, S > 1):
  * query s of row b sits at position pos[s] and sees cache slots j <= pos[s].

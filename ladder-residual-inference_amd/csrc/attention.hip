@@ -14,6 +14,7 @@
 // output in registers, K/V tiles of 32 keys broadcast from LDS as fp32).  Both: exact fp32
 // softmax semantics, one rounding of the output.
 #include "lr_common.h"
+#include <atomic>
 
 // ------------------------------------------------------------------------------------ decode
 static inline int attn_nsplit_cap(int Smax) {
@@ -265,6 +266,47 @@ extern "C" int lr_attn_decode(const void* q, int64_t ldq, const void* k_cache, c
   LR_DEC(64, 1) LR_DEC(64, 2) LR_DEC(64, 4) LR_DEC(64, 8)
 #undef LR_DEC
   return LR_E_UNSUPPORTED;
+}
+
+// ------------------------------------------------------------------------------------ decode, allocation-free
+// lr_attn_decode for callers that cannot allocate or carry a workspace: the split-KV partial
+// results live in a fixed device array of this library instead of caller memory.  `scratch` below
+// is, in host code, only a stand-in for the device symbol: the address kernels may use is looked
+// up once per device with hipGetSymbolAddress (every device holds its own copy of the array at
+// its own address) and kept in g_static_scratch; host code never passes `scratch` itself.
+constexpr size_t LR_STATIC_SCRATCH_BYTES = LR_ATTN_DECODE_STATIC_MAX_BYTES;
+constexpr int LR_MAX_DEVICES = 64;
+static __device__ __align__(256) unsigned char scratch[LR_STATIC_SCRATCH_BYTES];
+static std::atomic<float*> g_static_scratch[LR_MAX_DEVICES];
+
+// device address of `scratch` on the current device (looked up on the first call per device)
+static int static_scratch(float** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= LR_MAX_DEVICES) return LR_E_LAUNCH;
+  float* p = g_static_scratch[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    void* sym = nullptr;
+    if (hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)) != hipSuccess || sym == nullptr) {
+      (void)hipGetLastError();
+      return LR_E_LAUNCH;
+    }
+    p = reinterpret_cast<float*>(sym);
+    g_static_scratch[dev].store(p, std::memory_order_release);  // concurrent first calls store the same address
+  }
+  *out = p;
+  return LR_OK;
+}
+
+extern "C" int lr_attn_decode_static(const void* q, int64_t ldq, const void* k_cache, const void* v_cache,
+                                     const int32_t* pos, void* y, int64_t ldy, int B, int Hq, int Hkv, int hd,
+                                     int Smax, lr_stream_t stream) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || hd <= 0 || Smax <= 0) return LR_E_SHAPE;
+  const size_t need = lr_attn_decode_scratch_bytes(B, Hq, hd, Smax);
+  if (need > LR_STATIC_SCRATCH_BYTES) return LR_E_TOO_LARGE;
+  float* ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc != LR_OK) return rc;
+  return lr_attn_decode(q, ldq, k_cache, v_cache, pos, y, ldy, B, Hq, Hkv, hd, Smax, ws, need, stream);
 }
 
 // ------------------------------------------------------------------------------------ prefill

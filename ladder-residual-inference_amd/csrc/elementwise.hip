@@ -322,6 +322,7 @@ extern "C" const char* lr_error_string(int code) {
     case LR_E_SHAPE: return "non-positive or inconsistent size";
     case LR_E_UNSUPPORTED: return "size not supported by the gfx950 kernels";
     case LR_E_LAUNCH: return "HIP launch failed";
+    case LR_E_TOO_LARGE: return "the problem needs more scratch memory than the library's built-in buffer holds";
     default: return "unknown error code";
   }
 }

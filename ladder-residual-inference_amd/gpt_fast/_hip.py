@@ -29,6 +29,8 @@ _PROTOS = {
     "lr_attn_decode_scratch_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "lr_attn_decode": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int,
                                c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "lr_attn_decode_static": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,
+                                      c_int, c_int, c_int, c_void_p]),
     "lr_attn_prefill": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,
                                 c_int, c_int, c_int, c_int, c_void_p]),
     "lr_argmax": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_int, c_void_p]),
@@ -237,6 +239,20 @@ def attn_decode(q, k_cache, v_cache, pos, y, scratch, B, Hq, Hkv, hd):
     assert pos.dtype == torch.int32 and pos.numel() == 1 and scratch.dtype == torch.float32
     _check(load().lr_attn_decode(_dev(q), ldq, _dev(k_cache), _dev(v_cache), pos.data_ptr(), _dev(y), ldy, B, Hq, Hkv,
                                  hd, Smax, scratch.data_ptr(), scratch.numel() * 4, _stream()), "lr_attn_decode")
+    return y
+
+
+ATTN_DECODE_STATIC_MAX_BYTES = 32 << 20   # LR_ATTN_DECODE_STATIC_MAX_BYTES of include/ladder_hip.h
+
+
+def attn_decode_static(q, k_cache, v_cache, pos, y, B, Hq, Hkv, hd):
+    """lr_attn_decode with the partial results in the library's own fixed device array: nothing is allocated."""
+    _, _, ldq = _rows_ld(q)
+    _, _, ldy = _rows_ld(y)
+    Smax = k_cache.shape[2]
+    assert pos.dtype == torch.int32 and pos.numel() == 1
+    _check(load().lr_attn_decode_static(_dev(q), ldq, _dev(k_cache), _dev(v_cache), pos.data_ptr(), _dev(y), ldy, B, Hq,
+                                        Hkv, hd, Smax, _stream()), "lr_attn_decode_static")
     return y
 
 
