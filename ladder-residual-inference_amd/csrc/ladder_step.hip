@@ -5,23 +5,26 @@
 // ones (norms, RoPE, attention, combine) cost as much as the weight streaming.  Here one
 // workgroup per CU (512 lanes = 8 waves) stays resident for the whole step and walks the layers.
 //
-// The ladder schedule is what makes this wide: attention block t reads the residual stream
-// WITHOUT the MLP output of layer t-1 (in the reference that output is still inside an
-// all-reduce), so attention(t) and mlp(t-1) are independent and run side by side.  A "slot" t is,
-// per workgroup,
-//     residual adds + both RMSNorms (redundantly in every workgroup; the residual stream itself
-//         never leaves the workgroup's LDS)
-//     wqkv(t) rows
-//     attention workgroups (about one per 128 keys): attention(t) over their key range with K/V
-//         held in registers -- scores on the matrix cores (v_mfma_f32_32x32x16_bf16, one tile per
-//         32 keys), fp32 softmax and P.V -- un-normalised partial results; then each of them
-//         merges all partial results for its share of the output elements and publishes bf16
+// The ladder schedule is what makes this wide: attention(t) and mlp(t) both read the residual
+// stream BEFORE the other's output has been added (in the reference both outputs are still inside
+// an all-reduce at that point), so the two modules of a layer are independent and run side by
+// side.  A "slot" t = layer t is, per workgroup,
+//     R += a(t-1), attention norm (redundantly in every workgroup; the residual stream itself
+//         never leaves the workgroup's LDS); wqkv(t) rows
+//     attention workgroups (about one per 128 keys): R += m(t-1), then attention(t) over their key
+//         range with K/V held in registers -- scores on the matrix cores (v_mfma_f32_32x32x16_bf16,
+//         one tile per 32 keys), fp32 softmax and P.V -- un-normalised partial results; then each of
+//         them merges all partial results for its share of the output elements and publishes bf16
 //         words (every workgroup merging every partial itself costs 32 times the coherent reads,
 //         and those are what makes stragglers)
-//     all other workgroups: the scaling of the MLP input, left out of the norms above, then
-//         w1(t-1) rows + SwiGLU  (17 us of streaming that hides the attention latency chain)
-//     read the merged attention output, wo(t) rows
-//     w2(t-1) rows
+//     all other workgroups: R += m(t-1), ffn norm, w1(t) rows + SwiGLU  (15 us of streaming that
+//         hides the attention latency chain)
+//     read the merged attention output, wo(t) rows -> a(t)
+//     read the activations, w2(t) rows -> m(t)
+// Every hand-over between workgroups has independent streaming between its producer and its
+// consumer: a(t-1) is written by wo(t-1) and read after w2(t-1); m(t-1) is written by w2(t-1) and
+// read after the attention norm and wqkv(t); qkv(t) and the attention output are covered by w1(t);
+// the activations of w1(t) by wo(t).
 //
 // No barriers, flags or fences: everything that crosses workgroups (module outputs a / m, qkv,
 // activations, attention partials, argmax candidates) is exchanged as self-validating 32-bit
@@ -30,10 +33,9 @@
 // non-coherent per-XCD L2 lines.  A consumer optimistically loads what it needs and retries the
 // words whose tag is not yet the expected one, so a value is consumed the moment it lands and a
 // producer never waits.  Overwriting a word is safe once every workgroup has finished reading its
-// previous value; that is implied by data flow (nobody can produce slot t+1's qkv before slot
-// t's partials existed, ...) except for a / m / partials, for which every workgroup publishes a
-// "done" word after its residual bookkeeping and the attention workgroups -- through which all
-// later writes of the slot depend -- check all of them while they wait for q anyway.
+// previous value; that is implied by data flow alone (the chain is spelled out at the layer loop:
+// e.g. a(t) is written in wo(t), which needs the merged attention output, which needs all of
+// qkv(t), which every workgroup produces after it has read a(t-1)).
 // The values stored are bf16-representable, i.e. rounded exactly where the eager reference
 // rounds (fp32 attention partials take two words).  Weights, KV cache and logits use ordinary
 // accesses (read-only, or produced for the next launch).
@@ -78,8 +80,14 @@ constexpr int ATT_NI = 9;         // key iterations an attention wave keeps in r
 constexpr int NA_MAX = 16;        // attention workgroups (each merges a share of the outputs)
 constexpr int PROF_SLOTS = 4, PROF_POINTS = 16;
 // Buffer cache policies (the `aux` operand of the raw buffer builtins: bit 0 sc0, bit 1 nt, bit 4 sc1).
-constexpr int AUX_SC1 = 16;  // exchange stores: written through, visible to every XCD
-constexpr int AUX_LD = 17;   // exchange loads: sc0 sc1, never served from a per-XCD L2 line
+#ifndef LR_AUX_ST
+#define LR_AUX_ST 16
+#endif
+constexpr int AUX_SC1 = LR_AUX_ST;  // exchange stores: written through, visible to every XCD
+#ifndef LR_AUX_LD
+#define LR_AUX_LD 17
+#endif
+constexpr int AUX_LD = LR_AUX_LD;   // exchange loads: sc0 sc1, never served from a per-XCD L2 line
 constexpr int AUX_W = 2;     // weight loads: non-temporal (measured: nt on the exchange words' loads or stores is far slower)
 constexpr int POLL_SLEEP = 2;
 
@@ -109,7 +117,7 @@ struct StepParams {
   int hist_len, pos0, advance;
   unsigned char* ws;  // workspace base (Ctrl at offset 0)
   unsigned ws_bytes;
-  unsigned oa, om, oqkv, oact, oopart, omlpart, ocand, odone, oy;  // exchange buffers, offsets in 32-bit words
+  unsigned oa, om, oqkv, oact, oopart, omlpart, ocand, oy;  // exchange buffers, offsets in 32-bit words
   unsigned long long* prof;  // optional [nwg][PROF_SLOTS][PROF_POINTS] wall-clock stamps (100 MHz)
   int prof_t0;
 };
@@ -429,27 +437,6 @@ __device__ __forceinline__ Job load_job(const int* table, int kind, int wave, co
   return j;
 }
 
-// The jobs of slot t.  kind: 0 wqkv(t), 1 w1(t-1), 2 wo(t), 3 w2(t-1), 4 lm_head; a slot without
-// that module gets a job that owns no rows.  w1 is dealt to the workgroups that do not run
-// attention in the slot.
-__device__ __forceinline__ Job slot_job(const StepParams& p, const int* table, const u32* lring, int kind, int t,
-                                        int wave) {
-  const bool a = t < p.L, b = t >= 1 && t <= p.L;
-  int jk = JK_NONE, layer = 0, field = 0;
-  if (kind == 0 && a) { jk = JK_QKV; layer = t; field = LP_WQKV; }
-  if (kind == 1 && b) { jk = a ? JK_W1_SPLIT : JK_W1_ALL; layer = t - 1; field = LP_W1; }
-  if (kind == 2 && a) { jk = JK_WO; layer = t; field = LP_WO; }
-  if (kind == 3 && b) { jk = JK_W2; layer = t - 1; field = LP_W2; }
-  const u16* W = ring_ptr(lring, layer, field);
-  if (jk == JK_NONE) W = nullptr;
-  if (kind == 4) { jk = JK_HEAD; W = p.out_w; }
-  return load_job(table, jk, wave, W);
-}
-// first job of slot t + 1
-__device__ __forceinline__ Job next_slot_job(const StepParams& p, const int* table, const u32* lring, int t, int wave) {
-  return slot_job(p, table, lring, t + 1 < p.L ? 0 : (t + 1 == p.L ? 1 : 4), t + 1, wave);
-}
-
 struct Unit {
   u32x4_t r[RB];
 };
@@ -695,47 +682,70 @@ __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, con
 }
 
 // ------------------------------------------------------------------------------------------------
-// Residual bookkeeping + RMSNorm for the coming jobs, done redundantly by every workgroup (each
-// keeps its own copy of the residual stream in LDS, so only module outputs are ever exchanged):
-//   v1 = R (+ d1);  v2 = v1 (+ d2);  each add rounded to bf16;  R <- v2.
-//   x1 = norm(v1) * g1 -> LDS (if g1);  x2 = norm(v2) * g2 -> LDS (if g2).
-// At the first slot R comes from rows of the bf16 embedding table.  d1/d2 are tagged exchange
+// Residual bookkeeping + RMSNorm for the coming job, done redundantly by every workgroup (each keeps
+// its own copy of the residual stream in LDS, so only module outputs are ever exchanged):
+//   R <- bf16(R + d1) (if has_d1);  R <- bf16(R + d2) (if has_d2);  x = norm(R) * gain -> LDS (if gain).
+// At the first slot R comes from rows of the bf16 embedding table.  d1 / d2 are tagged exchange
 // arrays; all their loads are issued before the first one is checked.
 // ------------------------------------------------------------------------------------------------
 constexpr int PRO_NIT = 4;  // 8-element chunks per lane and row: dim <= PRO_NIT * NT * 8
+constexpr int EARLY_NIT = 2;  // chunks whose exchange words can be requested ahead of time (dim <= 8192 entirely)
+
+// The exchange words a coming residual_step will add (its d1), requested early -- before the job
+// that runs in between, or while that job's epilogue runs -- so that their round trip is over when
+// the step starts.  Words that were not there yet are polled by the step as usual.
+// (Batch 1 only: at batch 2 the 32 registers the words would occupy across a job are not there.)
 template <int M>
-struct LateNorm {  // what is needed to finish x1 after the phase that uses x2 (see prologue, finish_x1)
-  uint4 g[PRO_NIT];
-  float inv[M];
+struct EarlyWords {
+  static constexpr bool USED = M == 1;
+  u32x4_t r[1][EARLY_NIT][2];
 };
+// (every field is assigned on every path, `real` or not, so that the structure stays in registers; a
+// request that is not wanted goes out of the buffer's range and returns zero without touching memory)
+template <int M>
+__device__ __forceinline__ void issue_words(const Coh& coh, bool real, unsigned wo, int D, EarlyWords<M>& e) {
+  if (!EarlyWords<M>::USED) return;
+  const int tid = opaque_tid();
+#pragma unroll
+  for (int it = 0; it < EARLY_NIT; ++it) {
+    const int c = (it * NT + tid) * 8;
+    const unsigned o = (real && c < D) ? wo + (unsigned)c : 0x20000000u;
+    e.r[0][it][0] = coh.raw4(o);
+    e.r[0][it][1] = coh.raw4(o + 4u);
+  }
+}
 
 template <int M>
-__device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, u16* xr, const int* emb_rows,
-                                         bool has_d1, unsigned d1_wo, unsigned d1_tag, bool has_d2, unsigned d2_wo,
-                                         unsigned d2_tag, const u16* g1, const u16* g2, u16* x1, u16* x2, float* red,
-                                         const Job& first, Pipe& pipe, unsigned long long* stamp, LateNorm<M>& late,
-                                         bool defer1) {
+__device__ __forceinline__ void residual_step(const StepParams& p, const Coh& coh, u16* xr, const int* emb_rows,
+                                              bool has_d1, unsigned d1_wo, unsigned d1_tag, bool early1,
+                                              const EarlyWords<M>& e1, bool has_d2, unsigned d2_wo, unsigned d2_tag,
+                                              const u16* gain, u16* x, float* red, bool do_prime, const Job& first,
+                                              Pipe& pipe) {
   const int tid = opaque_tid(), D = p.D;
-  float ss1[M], ss2[M];
-  // the gains are needed only in pass 2 but are requested now: their latency hides behind pass 1
-  uint4 gq1[PRO_NIT], gq2[PRO_NIT];
+  float ss[M];
+  // the gain is needed only in pass 2 but is requested now: its latency hides behind pass 1
+  uint4 gq[PRO_NIT];
 #pragma unroll
   for (int it = 0; it < PRO_NIT; ++it) {
     const int c = (it * NT + tid) * 8;
-    gq1[it] = (g1 && c < D) ? ld16(g1 + c) : make_uint4(0, 0, 0, 0);
-    gq2[it] = (g2 && c < D) ? ld16(g2 + c) : make_uint4(0, 0, 0, 0);
+    gq[it] = (gain && c < D) ? ld16(gain + c) : make_uint4(0, 0, 0, 0);
   }
   // pass 1: the (bf16-exact) sums go to LDS unscaled; sums of squares per lane
 #pragma unroll
   for (int m = 0; m < M; ++m) {
-    ss1[m] = ss2[m] = 0.0f;
+    ss[m] = 0.0f;
     u32x4_t r1[PRO_NIT][2], r2[PRO_NIT][2];
 #pragma unroll
     for (int it = 0; it < PRO_NIT; ++it) {
       const int c = (it * NT + tid) * 8;
       if (c < D && has_d1) {
-        r1[it][0] = coh.raw4(d1_wo + m * D + c);
-        r1[it][1] = coh.raw4(d1_wo + m * D + c + 4);
+        if (EarlyWords<M>::USED && early1 && it < EARLY_NIT) {
+          r1[it][0] = e1.r[0][it < EARLY_NIT ? it : 0][0];
+          r1[it][1] = e1.r[0][it < EARLY_NIT ? it : 0][1];
+        } else {
+          r1[it][0] = coh.raw4(d1_wo + m * D + c);
+          r1[it][1] = coh.raw4(d1_wo + m * D + c + 4);
+        }
       }
       if (c < D && has_d2) {
         r2[it][0] = coh.raw4(d2_wo + m * D + c);
@@ -760,96 +770,49 @@ __device__ __forceinline__ void prologue(const StepParams& p, const Coh& coh, u1
 #pragma unroll
           for (int j = 0; j < 8; ++j) v[j] = round_bf(v[j] + t[j]);
         }
-        if (g1) st16(x1 + m * D + c, pack8(v));
-#pragma unroll
-        for (int j = 0; j < 8; ++j) ss1[m] += v[j] * v[j];
         if (has_d2) {
           bf4_from(coh.settle4(d2_wo + m * D + c, d2_tag, r2[it][0]), t);
           bf4_from(coh.settle4(d2_wo + m * D + c + 4, d2_tag, r2[it][1]), t + 4);
 #pragma unroll
           for (int j = 0; j < 8; ++j) v[j] = round_bf(v[j] + t[j]);
         }
-        if (g2) st16(x2 + m * D + c, pack8(v));
+        if (gain) st16(x + m * D + c, pack8(v));
 #pragma unroll
-        for (int j = 0; j < 8; ++j) ss2[m] += v[j] * v[j];
-        st16(xr + m * D + c, pack8(v));
+        for (int j = 0; j < 8; ++j) ss[m] += v[j] * v[j];
+        if (has_d1 || has_d2 || emb_rows) st16(xr + m * D + c, pack8(v));
       }
     }
   }
   // The first weight units of the coming job are requested only now, behind the exchange words: a
-  // wave's loads return in order and a CU serves them at a bounded rate, so requested at the end of
-  // the previous job they would stand between this phase and the words it waits for; from here they
-  // travel while the norms are finished.
-  if (stamp && tid == 0) stamp[12] = wall_clock64();
-  prime(first, tid & 63, pipe);
+  // wave's loads return in order and a CU serves them at a bounded rate, so requested earlier they
+  // would stand between this phase and the words it waits for; from here they travel while the
+  // norm is finished.
+  if (do_prime) prime(first, tid & 63, pipe);
+  if (gain == nullptr) return;  // uniform: only the residual was wanted (each lane revisits its own elements later)
 #pragma unroll
-  for (int m = 0; m < M; ++m) {
-    ss1[m] = wave_sum(ss1[m]);
-    ss2[m] = wave_sum(ss2[m]);
-  }
+  for (int m = 0; m < M; ++m) ss[m] = wave_sum(ss[m]);
   if ((tid & 63) == 0) {
 #pragma unroll
-    for (int m = 0; m < M; ++m) {
-      red[((tid >> 6) * M + m) * 2] = ss1[m];
-      red[((tid >> 6) * M + m) * 2 + 1] = ss2[m];
-    }
+    for (int m = 0; m < M; ++m) red[(tid >> 6) * M + m] = ss[m];
   }
   wg_sync();
-  if (stamp && tid == 0) stamp[13] = wall_clock64();
   // pass 2: scale in place (each lane revisits the elements it wrote)
 #pragma unroll
   for (int m = 0; m < M; ++m) {
-    float s1 = 0.0f, s2 = 0.0f;
+    float s1 = 0.0f;
 #pragma unroll
-    for (int wv = 0; wv < NW; ++wv) {
-      s1 += red[(wv * M + m) * 2];
-      s2 += red[(wv * M + m) * 2 + 1];
-    }
-    const float inv1 = rsqrtf(s1 / (float)D + p.eps), inv2 = rsqrtf(s2 / (float)D + p.eps);
-    late.inv[m] = inv1;
+    for (int wv = 0; wv < NW; ++wv) s1 += red[wv * M + m];
+    const float inv = rsqrtf(s1 / (float)D + p.eps);
 #pragma unroll
     for (int it = 0; it < PRO_NIT; ++it) {
       const int c = (it * NT + tid) * 8;
       if (c >= D) break;
       float v[8], g[8], o[8];
-      if (g1 && !defer1) {
-        unpack8(*reinterpret_cast<const uint4*>(x1 + m * D + c), v);
-        unpack8(gq1[it], g);
+      unpack8(*reinterpret_cast<const uint4*>(x + m * D + c), v);
+      unpack8(gq[it], g);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) o[j] = round_bf(v[j] * inv1) * g[j];
-        st16(x1 + m * D + c, pack8(o));
-      }
-      if (g2) {
-        unpack8(*reinterpret_cast<const uint4*>(x2 + m * D + c), v);
-        unpack8(gq2[it], g);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) o[j] = round_bf(v[j] * inv2) * g[j];
-        st16(x2 + m * D + c, pack8(o));
-      }
-    }
-  }
-#pragma unroll
-  for (int it = 0; it < PRO_NIT; ++it) late.g[it] = gq1[it];
-  wg_sync();
-}
-
-// The scaling of x1 that prologue() left out (defer1): x1 = round(v1 * inv) * g1, in place.  Only
-// the workgroups that use x1 call it, after the phase that needed x2 first.
-template <int M>
-__device__ __forceinline__ void finish_x1(const StepParams& p, u16* x1, const LateNorm<M>& late) {
-  const int tid = opaque_tid(), D = p.D;
-#pragma unroll
-  for (int m = 0; m < M; ++m) {
-#pragma unroll
-    for (int it = 0; it < PRO_NIT; ++it) {
-      const int c = (it * NT + tid) * 8;
-      if (c >= D) break;
-      float v[8], g[8], o[8];
-      unpack8(*reinterpret_cast<const uint4*>(x1 + m * D + c), v);
-      unpack8(late.g[it], g);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) o[j] = round_bf(v[j] * late.inv[m]) * g[j];
-      st16(x1 + m * D + c, pack8(o));
+      for (int j = 0; j < 8; ++j) o[j] = round_bf(v[j] * inv) * g[j];
+      st16(x + m * D + c, pack8(o));
     }
   }
   wg_sync();
@@ -916,7 +879,7 @@ __device__ __forceinline__ void attention_load(const StepParams& p, const LayerP
 
 template <int M, int HD, int G>
 __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh& coh, const LayerPtrs& lp, int b,
-                                                  int kvh, int k0, int k1, int pos, unsigned tag, bool poll_done,
+                                                  int kvh, int k0, int k1, int pos, unsigned tag,
                                                   unsigned long long* stamp,
                                                   KV<HD>& kv, u32* qp,
                                                   float* sc, int sc_ld, float* ored, u32* kp, float* vnew,
@@ -934,24 +897,15 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
   const unsigned o_out = p.oopart + (unsigned)((((b * Hq + kvh * G) * NA) + aw) * HD * 2);
   const unsigned ml_out = p.omlpart + (unsigned)((((b * Hq + kvh * G) * NA) + aw) * 4);
 
-  // ---- every workgroup has finished reading the previous slot's exchange data once its "done"
-  //      word carries this slot's tag: only then may partial results (and, downstream of them,
-  //      module outputs) be overwritten
   // Everything this phase waits for is requested at once; what has not landed yet is polled.
   const bool own = owner && tid < HD / 2;
   const unsigned ko = qkv + (unsigned)(Hq * HD + kvh * HD + 2 * tid), vo = ko + (unsigned)(Hkv * HD);
   const unsigned q0 = qkv + (unsigned)(kvh * G * HD + 2 * tid);  // pair `tid` of the G * HD / 2 pairs of this group
-  unsigned dr = 0;
   u32x2_t qr = {0u, 0u}, rk = {0u, 0u}, rv = {0u, 0u};
-  if (poll_done && tid < (int)gridDim.x) dr = coh.raw1(p.odone + (unsigned)tid);
   if (tid < G * HD / 2) qr = coh.raw2(q0);
   if (own) {
     rk = coh.raw2(ko);
     rv = coh.raw2(vo);
-  }
-  if (poll_done) {
-    if (tid < (int)gridDim.x && ((dr ^ tag) & 0xffffu) != 0) coh.poll1(p.odone + (unsigned)tid, tag);
-    for (int i = tid + NT; i < (int)gridDim.x; i += NT) coh.poll1(p.odone + (unsigned)i, tag);
   }
   // ---- rotate q (all G heads) into LDS; the owner of `pos` also rotates k, keeps k/v in LDS and
   //      writes them to the cache for the following steps
@@ -979,7 +933,7 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
     *reinterpret_cast<u32*>(lp.v_cache + slot) = pack_bf2(v0, v1);
   }
   wg_sync();
-  if (stamp && tid == 0) stamp[8] = wall_clock64();
+  if (stamp && tid == 0) stamp[10] = wall_clock64();
   if (n <= 0) {
     for (int i = tid; i < G * HD; i += NT)
       coh.st_f32(o_out + (unsigned)(((i / HD) * NA * HD + (i % HD)) * 2), 0.0f, tag);
@@ -1022,7 +976,7 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
     }
   }
   wg_sync();
-  if (stamp && tid == 0) stamp[9] = wall_clock64();
+  if (stamp && tid == 0) stamp[11] = wall_clock64();
   // ---- softmax statistics: a wave per head; sc becomes exp(s - max)
   for (int g = wave; g < G; g += NW) {
     float m = -INFINITY;
@@ -1038,7 +992,7 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
     if (lane == 0) { s_m[g] = m; s_l[g] = l; }
   }
   wg_sync();
-  if (stamp && tid == 0) stamp[10] = wall_clock64();
+  if (stamp && tid == 0) stamp[12] = wall_clock64();
   // ---- P.V: GB heads at a time share the unpacked V rows; the key groups of a wave are folded with
   //      lane-half / lane-row swaps (one swap + one add folds two accumulators), the waves in LDS
   constexpr int GB = G < 8 ? G : 8;
@@ -1169,7 +1123,7 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   u16* xb = xa + xlen;                                  // MLP-chain input        [M][<= max(D, I)]
   u16* xr = xb + xlen;                                  // residual stream        [M][D]
   float* part = reinterpret_cast<float*>(xr + M * D);   // [NW][NJMAX * M]
-  float* red = part + NW * NJMAX * M;                   // [NW][M][2]
+  float* red = part + NW * NJMAX * M;                   // [NW][M] (space for [NW][M][2])
   float* qs = red + NW * M * 2;                         // [G][HD / 2] packed bf16 pairs (space for [G][HD])
   float* sc = qs + G * HD;                              // [G][sc_ld]
   float* ored = sc + G * sc_ld;                         // [NW][G][HD]
@@ -1219,86 +1173,118 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
 
   const int qdim = Hq * HD;
   Pipe pipe;
-  LateNorm<M> late;
 
+#ifdef LR_STEP_PROFILE
 #define LR_STAMP(k)                                                                                  \
   if (p.prof && t >= p.prof_t0 && t < p.prof_t0 + PROF_SLOTS && tid == 0)                            \
     p.prof[((size_t)blockIdx.x * PROF_SLOTS + (t - p.prof_t0)) * PROF_POINTS + (k)] = wall_clock64();
-#define LR_JOB(kind) slot_job(p, jtab, lring, kind, t, wave)
-  for (int t = 0; t <= L; ++t) {
-    const bool has_a = t < L, has_b = t >= 1;
+#define LR_STAMP_PTR                                                                                 \
+  ((p.prof && t >= p.prof_t0 && t < p.prof_t0 + PROF_SLOTS)                                          \
+       ? p.prof + ((size_t)blockIdx.x * PROF_SLOTS + (t - p.prof_t0)) * PROF_POINTS : nullptr)
+#else
+#define LR_STAMP(k)
+#define LR_STAMP_PTR nullptr
+#endif
+#define LR_JOB(jk, field) load_job(jtab, jk, wave, ring_ptr(lring, t, field))
+  const Job no_job = load_job(jtab, JK_NONE, wave, nullptr);
+  const Job j_head = load_job(jtab, JK_HEAD, wave, p.out_w);
+  // Slot t = layer t: attention(t) and mlp(t) both read the residual stream before the other's
+  // output is added (the ladder schedule: in the reference both outputs are in flight in an
+  // all-reduce at that point), so they run side by side.  Order of the hand-overs in a slot, each
+  // with independent streaming between producer and consumer:
+  //   a(t-1) [written by wo(t-1), then w2(t-1) streamed]      -> residual + attention norm -> wqkv(t)
+  //   m(t-1) [written by w2(t-1), then the norm and wqkv(t)]  -> residual + ffn norm       -> w1(t)
+  //   qkv(t) -> attention(t) on NA workgroups while the others stream w1(t) -> merged y(t) -> wo(t)
+  //   act(t) [written by w1(t), then wo(t) streamed]          -> w2(t)
+  // The m words are requested a phase ahead, before wqkv's rows, and w1's first weight units go out at
+  // the end of wqkv: the ffn norm then finds its words there and w1 its first units.  (The same for the
+  // a words -- requested while w2's epilogue runs -- is slower: they are often not all written yet, and a
+  // word found stale costs a second dependent round trip.)
+  // Overwriting an exchange array is safe by data flow alone: e.g. a(t) is written in wo(t), which
+  // needs all of y(t), which needs every attention workgroup's merge, which needs all of qkv(t),
+  // which every workgroup produces after it has read a(t-1); likewise for m (through act(t) and,
+  // for the attention workgroups, y(t)), qkv, the partial results, y and act.
+  // (The loop is rotated: the residual step that opens slot t + 1 sits at the END of iteration t, so
+  // that it and the closing step after the last layer are one piece of code.)
+  EarlyWords<M> ew;
+  issue_words<M>(coh, false, 0u, D, ew);
+  // ---------------- slot 0 opens with R = embedding rows; attention norm; the first weight units of wqkv(0)
+  residual_step<M>(p, coh, xr, p.tokens, false, 0u, 0u, false, ew, false, 0u, 0u, ring_ptr(lring, 0, LP_ATTN_NORM), xa, red,
+                   true, load_job(jtab, JK_QKV, wave, ring_ptr(lring, 0, LP_WQKV)), pipe);
+  for (int t = 0; t < L; ++t) {
     // request the pointer record of layer t + 2 now; it goes into the ring at the end of the slot
     u32 ring_next = 0;
     if (tid < 16 && t + 2 < L) ring_next = reinterpret_cast<const u32*>(p.layers + t + 2)[tid];
     const unsigned tag = tag_of(epoch_base + (unsigned)t + 1u), tag_prev = tag_of(epoch_base + (unsigned)t);
     const unsigned act_wo = p.oact + (unsigned)((t & 1) * M * I);  // activations alternate between two buffers
-    LR_STAMP(0)
-    // ---------------- v1 = R + m(t-2) feeds mlp(t-1); v2 = v1 + a(t-1) feeds attention(t)
-    prologue<M>(p, coh, xr, t == 0 ? p.tokens : nullptr, t >= 2, p.om, tag_prev, t >= 1 && has_a, p.oa, tag_prev,
-                has_b ? ring_ptr(lring, t - 1, LP_FFN_NORM) : nullptr,
-                has_a ? ring_ptr(lring, t, LP_ATTN_NORM) : nullptr, xb, xa, red, LR_JOB(has_a ? 0 : 1), pipe,
-                (p.prof && t >= p.prof_t0 && t < p.prof_t0 + PROF_SLOTS)
-                    ? p.prof + ((size_t)blockIdx.x * PROF_SLOTS + (t - p.prof_t0)) * PROF_POINTS
-                    : nullptr,
-                late, has_a && has_b);
-    // this workgroup no longer reads a / m / the previous partials
-    if (tid == 0) coh.st(p.odone + (unsigned)w, 0.0f, tag);
     LR_STAMP(1)
-    if (has_a && att_wg) {
-      run_job<M, EPI_STORE>(p, coh, LR_JOB(0), LR_JOB(2), pipe, xa, part, p.oqkv, p.nqkv, tag, nullptr, nullptr,
-                            nullptr, nullptr);
+    const Job j_qkv = LR_JOB(JK_QKV, LP_WQKV);
+    // m(t-1) for the coming residual step: on its way while the query/key/value rows are done
+    issue_words<M>(coh, t >= 1, p.om, D, ew);
+    if (att_wg) {
+      // (no weight units are requested across the attention phase: it is where registers are scarcest, and
+      // the attention workgroups are done well before the others have streamed w1)
+      run_job<M, EPI_STORE>(p, coh, j_qkv, no_job, pipe, xa, part, p.oqkv, p.nqkv, tag, nullptr, nullptr, nullptr,
+                            nullptr);
       LR_STAMP(2)
-      // ---------------- attention workgroup (it owns no rows of w1)
+      // ---------------- attention workgroup (it owns no rows of w1): R += m(t-1) while q is on its way
+      if (t >= 1)
+        residual_step<M>(p, coh, xr, nullptr, true, p.om, tag_prev, true, ew, false, 0u, 0u, nullptr, xb, red, false,
+                         no_job, pipe);
+      LR_STAMP(3)
       KV<HD> kv;
       LayerPtrs lcache;  // only the cache pointers are used
       lcache.k_cache = const_cast<u16*>(ring_ptr(lring, t, LP_K_CACHE));
       lcache.v_cache = const_cast<u16*>(ring_ptr(lring, t, LP_V_CACHE));
-      bool first = true;
       for (int b = 0; b < p.B; ++b)
         for (int kvh = 0; kvh < p.Hkv; ++kvh) {
           attention_load<HD>(p, lcache, b, kvh, k0, k1, pos, kv);
-          attention_compute<M, HD, G>(p, coh, lcache, b, kvh, k0, k1, pos, tag, first,
-                                      (p.prof && t >= p.prof_t0 && t < p.prof_t0 + PROF_SLOTS)
-                                          ? p.prof + ((size_t)blockIdx.x * PROF_SLOTS + (t - p.prof_t0)) * PROF_POINTS
-                                          : nullptr,
-                                      kv, reinterpret_cast<u32*>(qs), sc, sc_ld, ored, reinterpret_cast<u32*>(knew), vnew, s_m, s_l);
-          first = false;
+          attention_compute<M, HD, G>(p, coh, lcache, b, kvh, k0, k1, pos, tag, LR_STAMP_PTR, kv,
+                                      reinterpret_cast<u32*>(qs), sc, sc_ld, ored, reinterpret_cast<u32*>(knew), vnew,
+                                      s_m, s_l);
         }
       attention_merge_slice<M, HD>(p, coh, Hq, tag, wbuf, w);
+      prime(LR_JOB(JK_WO, LP_WO), opaque_tid() & 63, pipe);
     } else {
-      run_job<M, EPI_STORE>(p, coh, LR_JOB(0), LR_JOB(1), pipe, xa, part, p.oqkv, p.nqkv, tag, nullptr, nullptr,
-                            nullptr, nullptr);
+      const Job j_w1 = LR_JOB(JK_W1_SPLIT, LP_W1);
+      run_job<M, EPI_STORE>(p, coh, j_qkv, j_w1, pipe, xa, part, p.oqkv, p.nqkv, tag, nullptr, nullptr, nullptr,
+                            nullptr);
       LR_STAMP(2)
-      if (has_a && has_b) finish_x1<M>(p, xb, late);  // its first weight units are on their way meanwhile
-      // ---------------- everyone else: the up/gate projection of the previous layer + SwiGLU
-      const Job after_w1 = LR_JOB(has_a ? 2 : 3);  // named values, not conditional temporaries: they stay in registers
-      run_job<M, EPI_SWIGLU>(p, coh, LR_JOB(1), after_w1, pipe, xb, part, act_wo, I, tag, nullptr, nullptr, nullptr,
+      // ---------------- everyone else: R += m(t-1); ffn norm; the up/gate projection + SwiGLU
+      residual_step<M>(p, coh, xr, nullptr, t >= 1, p.om, tag_prev, t >= 1, ew, false, 0u, 0u,
+                       ring_ptr(lring, t, LP_FFN_NORM), xb, red, false, no_job, pipe);
+      LR_STAMP(3)
+      run_job<M, EPI_SWIGLU>(p, coh, j_w1, LR_JOB(JK_WO, LP_WO), pipe, xb, part, act_wo, I, tag, nullptr, nullptr, nullptr,
                              nullptr);
     }
-    LR_STAMP(3)
+    LR_STAMP(4)
     // ---------------- merged attention output (published by the attention workgroups), output projection
-    if (has_a) {
-      load_x<M>(coh, p.oy, tag, qdim, xa);
-      LR_STAMP(4)
-      Job after_wo = slot_job(p, jtab, lring, -1, 0, wave);
-      if (has_b) after_wo = LR_JOB(3);
-      run_job<M, EPI_STORE>(p, coh, LR_JOB(2), after_wo, pipe, xa, part, p.oa, D, tag, nullptr, nullptr, nullptr,
-                            nullptr);
-    } else if (has_b) {
-      // no attention in this slot, hence nobody has checked the "done" words yet: do it here,
-      // before the down projection overwrites m
-      for (int i = tid; i < nwg; i += NT) coh.poll1(p.odone + (unsigned)i, tag);
-    }
+    load_x<M>(coh, p.oy, tag, qdim, xa);
     LR_STAMP(5)
-    // ---------------- down projection of the previous layer
-    if (has_b) {
-      load_x<M>(coh, act_wo, tag, I, xb);
-      LR_STAMP(6)
-      run_job<M, EPI_STORE>(p, coh, LR_JOB(3), slot_job(p, jtab, lring, -1, 0, wave), pipe, xb, part, p.om, D, tag,
-                            nullptr, nullptr, nullptr, nullptr);
-    }
+    run_job<M, EPI_STORE>(p, coh, LR_JOB(JK_WO, LP_WO), LR_JOB(JK_W2, LP_W2), pipe, xa, part, p.oa, D, tag, nullptr,
+                          nullptr, nullptr, nullptr);
+    LR_STAMP(6)
+    // ---------------- down projection
+    load_x<M>(coh, act_wo, tag, I, xb);
     LR_STAMP(7)
-    if (tid < 16 && t + 2 < L) lring[((t + 2) & 3) * 16 + tid] = ring_next;
+    run_job<M, EPI_STORE>(p, coh, LR_JOB(JK_W2, LP_W2), no_job, pipe, xb, part, p.om, D, tag, nullptr, nullptr, nullptr,
+                          nullptr);
+    LR_STAMP(8)
+    // ---------------- slot t + 1 opens: R += a(t); attention norm; the first weight units of wqkv(t + 1) go out
+    //                  behind the a words.  After the last layer: x = (R + a(L-1)) + m(L-1), the final norm and
+    //                  the first units of the lm_head instead.
+    {
+      const bool last = t + 1 == L;
+      Job j_first = j_head;
+      if (!last) j_first = load_job(jtab, JK_QKV, wave, ring_ptr(lring, t + 1, LP_WQKV));
+      residual_step<M>(p, coh, xr, nullptr, true, p.oa, tag, false, ew, last, p.om, tag,
+                       last ? p.final_norm : ring_ptr(lring, t + 1, LP_ATTN_NORM), xa, red, true, j_first, pipe);
+    }
+    LR_STAMP(0)
+    {
+      const int rt = opaque_tid();  // (not hoisted out of the loop and spilled: a scratch reload waits for every load in flight)
+      if (rt < 16 && t + 2 < L) lring[((t + 2) & 3) * 16 + rt] = ring_next;
+    }
     // one workgroup-wide look at the failure flag per slot keeps a broken step from running on
     if (tid == 0) s_flag[0] = (int)cldu(&ctrl->fail);
     wg_sync();
@@ -1306,15 +1292,12 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   }
 #undef LR_JOB
 #undef LR_STAMP
-  // ---------------- head: x = (R + a(L-1)) + m(L-1), final norm, vocab-shard lm_head, argmax
-  const unsigned tag = tag_of(epoch_base + (unsigned)L + 2u), tag_prev = tag_of(epoch_base + (unsigned)L + 1u);
-  prologue<M>(p, coh, xr, nullptr, true, p.oa, tag_of(epoch_base + (unsigned)L), true, p.om, tag_prev, nullptr,
-              p.final_norm, xb, xa, red, slot_job(p, jtab, lring, 4, L + 1, wave), pipe, nullptr, late, false);
+#undef LR_STAMP_PTR
+  // ---------------- head: vocab-shard lm_head on the normed x, argmax
+  const unsigned tag = tag_of(epoch_base + (unsigned)L + 1u);
   float best_v = -INFINITY;
   int best_i = 0x7fffffff;
-  run_job<M, EPI_LOGITS>(p, coh, slot_job(p, jtab, lring, 4, L + 1, wave), slot_job(p, jtab, lring, -1, 0, wave), pipe,
-                         xa, part, 0u, 0, tag,
-                         cand_v, cand_i, &best_v, &best_i);
+  run_job<M, EPI_LOGITS>(p, coh, j_head, no_job, pipe, xa, part, 0u, 0, tag, cand_v, cand_i, &best_v, &best_i);
   if (tid < M) {  // candidate: value (bf16-exact), a filler word, index as two 16-bit halves
     const unsigned wo = p.ocand + (unsigned)((w * M + tid) * 4);
     coh.st(wo, best_v, tag);
@@ -1370,7 +1353,7 @@ __global__ void k_step_init(Ctrl* c, unsigned nwg, unsigned* words, unsigned n_w
 }
 
 struct Layout {
-  size_t ctrl, abuf, mbuf, qkv, act, opart, mlpart, cand, done, y, total;
+  size_t ctrl, abuf, mbuf, qkv, act, opart, mlpart, cand, y, total;
 };
 
 static int num_cus() {
@@ -1425,16 +1408,19 @@ static Layout make_layout(const lr_ladder_model_t* md, int B, int nwg) {
   l.opart = o; o = up(o + 4 * (size_t)B * Hq * na * hd * 2);
   l.mlpart = o; o = up(o + 4 * (size_t)B * Hq * na * 4);
   l.cand = o; o = up(o + 4 * (size_t)nwg * B * 4);
-  l.done = o; o = up(o + 4 * (size_t)nwg);
   l.y = o; o = up(o + 4 * (size_t)B * Hq * hd);
   l.total = o;
   return l;
 }
 
 // (batch, head_dim, q heads per kv head) combinations the step kernel is instantiated for
+#ifdef LR_STEP_ONLY_70B  // experiments: one instance compiles in a fraction of the time
+#define LR_STEP_INSTANCES(X) X(1, 128, 8)
+#else
 #define LR_STEP_INSTANCES(X) \
   X(1, 128, 8) X(2, 128, 8) X(1, 128, 4) X(2, 128, 4) X(1, 64, 4) X(2, 64, 4) X(1, 128, 16) \
   X(1, 64, 2) X(2, 64, 2) X(1, 128, 2) X(1, 128, 1) X(1, 64, 1) X(1, 64, 8)
+#endif
 
 static bool has_instance(int B, int hd, int G) {
 #define LR_HAS(MV, HDV, GV) if (B == MV && hd == HDV && G == GV) return true;
@@ -1473,6 +1459,7 @@ static int validate(const lr_ladder_model_t* md, int B) {
   if (lds_need(B, md->head_dim, G, md->dim, md->ffn, md->n_head) > 160 * 1024) return LR_E_UNSUPPORTED;
   const int nwg = num_cus();
   if (nwg < 2) return LR_E_LAUNCH;
+  if (md->dim > NJMAX * nwg) return LR_E_UNSUPPORTED;  // a workgroup's rows of wo / w2 fit one reduction round
   const int na = pick_na(md->smax, md->head_dim, nwg, md->attention_workgroups);
   if (na > NA_MAX || (md->smax + na - 1) / na > att_capacity(md->head_dim)) return LR_E_UNSUPPORTED;
   if (!md->tok_embeddings || !md->norm || !md->output || !md->freqs_cis || !md->layers_dev) return LR_E_NULL;
@@ -1563,7 +1550,7 @@ extern "C" int lr_ladder_decode_step(const lr_ladder_model_t* md, int batch, con
   sp.oa = (unsigned)(l.abuf / 4); sp.om = (unsigned)(l.mbuf / 4);
   sp.oqkv = (unsigned)(l.qkv / 4); sp.oact = (unsigned)(l.act / 4);
   sp.oopart = (unsigned)(l.opart / 4); sp.omlpart = (unsigned)(l.mlpart / 4); sp.ocand = (unsigned)(l.cand / 4);
-  sp.odone = (unsigned)(l.done / 4); sp.oy = (unsigned)(l.y / 4);
+  sp.oy = (unsigned)(l.y / 4);
 #ifdef LR_STEP_PROFILE
   sp.prof = g_prof;
   sp.prof_t0 = g_prof_t0;
