@@ -97,6 +97,21 @@ int lr_linear(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, i
 int lr_linear_tuned(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
                     int act_swiglu, int gemv_cfg, lr_stream_t stream);
 
+/* Weight-only fp8 linear:  y[m, n] = bf16( bf16( sum_k x[m, k] * w8[n, k] ) * scales[n] ).
+ * w8 [N, K] dense float8 e4m3 (OCP "e4m3fn": bias 7, no infinities, max 448), one byte per weight;
+ * scales [N] bf16, one per output row; x, y bf16 as in lr_linear.  K % 16 == 0.
+ * The reference leaves the hook of gpt-fast's weight-only quantised layers -- a Linear replacement
+ * holding `weight` in the narrow type and `scales` in the model dtype (gpt_ladder_TP.py:233-237) --
+ * whose forward is F.linear(x, weight.to(x.dtype)) * scales; this is that forward with e4m3 weights
+ * (the reference ships no quantiser and no quantised layer, so parity at this boundary is pinned by
+ * the formula only).  M <= 8 (decode) streams the fp8 weights once: half the HBM bytes of lr_linear.
+ * M > 8 (prefill) expands the weights to bf16 into `scratch` (lr_linear_fp8_scratch_bytes(M, N, K)
+ * bytes, 16-byte aligned), runs lr_linear on them and scales the columns; scratch may be NULL for
+ * M <= 8. */
+size_t lr_linear_fp8_scratch_bytes(int M, int N, int K);
+int lr_linear_fp8(const void* x, int64_t ldx, const void* w8, const void* scales, void* y, int64_t ldy, int M, int N,
+                  int K, void* scratch, size_t scratch_bytes, lr_stream_t stream);
+
 /* out[r, i] = bf16( bf16(silu(h[r, I + i])) * h[r, i] ),  h [rows, 2I] = [u | g] (row stride ldh).
  * F.silu(g) * u after chunk(2), utils.py:147-148 and :386. */
 int lr_swiglu(const void* h, int64_t ldh, void* out, int rows, int I, lr_stream_t stream);

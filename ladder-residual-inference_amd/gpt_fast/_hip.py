@@ -23,6 +23,9 @@ _PROTOS = {
     "lr_linear": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
     "lr_linear_tuned": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int,
                                 c_void_p]),
+    "lr_linear_fp8_scratch_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "lr_linear_fp8": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p,
+                              c_size_t, c_void_p]),
     "lr_swiglu": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_int, c_void_p]),
     "lr_rope_kv_write": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                  c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
@@ -160,6 +163,31 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, act_swiglu: bool
     return out
 
 
+_FP8_SCRATCH = {}
+
+
+def linear_fp8(x: torch.Tensor, w8: torch.Tensor, scales: torch.Tensor, out: torch.Tensor):
+    """out[M, N] = (x[M, K] @ w8[N, K]^T rounded to bf16) * scales[N]: weight-only e4m3 linear.  For M > 8 the
+    expanded weights go through a per-device scratch buffer that grows to the largest matrix seen (allocated
+    here, outside the library; allocate it before capturing a graph by running the shape once)."""
+    M, K, ldx = _rows_ld(x)
+    N, Kw = w8.shape
+    assert w8.dtype == torch.float8_e4m3fn and w8.is_contiguous() and Kw == K and w8.is_cuda
+    assert scales.dtype == torch.bfloat16 and scales.numel() == N and scales.is_contiguous()
+    Mo, No, ldy = _rows_ld(out)
+    assert (Mo, No) == (M, N), (out.shape, M, N)
+    lib = load()
+    need = int(lib.lr_linear_fp8_scratch_bytes(M, N, K))
+    scratch = None
+    if need:
+        scratch = _FP8_SCRATCH.get(x.device)
+        if scratch is None or scratch.numel() < need:
+            scratch = _FP8_SCRATCH[x.device] = torch.empty(need, dtype=torch.uint8, device=x.device)
+    _check(lib.lr_linear_fp8(_dev(x), ldx, w8.data_ptr(), _dev(scales), _dev(out), ldy, M, N, K,
+                             None if scratch is None else scratch.data_ptr(), need, _stream()), "lr_linear_fp8")
+    return out
+
+
 def linear_swiglu(h: torch.Tensor, w: torch.Tensor, out: torch.Tensor, act: torch.Tensor = None):
     """out = (silu(g) * u) @ w^T for h = [u | g].  Up to 4 rows the activation is fused into the
     weight-streaming GEMV; above that it is materialised once (in `act`, or a new tensor) and fed to
@@ -171,6 +199,26 @@ def linear_swiglu(h: torch.Tensor, w: torch.Tensor, out: torch.Tensor, act: torc
         act = h.new_empty(M, two_k // 2)
     swiglu(h, act)
     return linear(act, w, out)
+
+
+def module_linear(x: torch.Tensor, mod, out: torch.Tensor):
+    """mod(x) for an nn.Linear (bf16 weight) or a weight-only fp8 replacement (`weight` e4m3 + `scales`)."""
+    scales = getattr(mod, "scales", None)
+    if scales is not None:
+        return linear_fp8(x, mod.weight, scales, out)
+    return linear(x, mod.weight, out)
+
+
+def module_linear_swiglu(h: torch.Tensor, mod, out: torch.Tensor, act: torch.Tensor = None):
+    """mod(silu(g) * u) for h = [u | g]."""
+    scales = getattr(mod, "scales", None)
+    if scales is None:
+        return linear_swiglu(h, mod.weight, out, act)
+    M, two_k, _ = _rows_ld(h)
+    if act is None:
+        act = h.new_empty(M, two_k // 2)
+    swiglu(h, act)
+    return linear_fp8(act, mod.weight, scales, out)
 
 
 def swiglu(h: torch.Tensor, out: torch.Tensor):

@@ -33,7 +33,7 @@ class Workspace:
         self.qkv = e(rows, fused_width)
         self.y = e(rows, cfg.n_head_local * hd)
         self.h = e(rows, 2 * cfg.ffn_local)
-        self.act = e(rows, cfg.ffn_local) if rows > 4 else None   # activated MLP input for the GEMM path
+        self.act = e(rows, cfg.ffn_local)   # activated MLP input where SwiGLU is not fused into the projection
         self.logits = e(B, S if all_logits else 1, cfg.output_rows)
         self.next_token = torch.empty(B, 1, dtype=torch.int32, device=device)
         self.next_token_valid_for = None   # set by a fused decode step that already chose the token
@@ -93,6 +93,9 @@ class GPTBase(nn.Module):
         self.max_seq_length = max_seq_length
         self.max_batch_size = max_batch_size
         dtype = self.output.weight.dtype
+        # for weight-only quantised layers the model dtype is the scales' (gpt_ladder_TP.py:232-237)
+        if hasattr(self.output, "scales"):
+            dtype = self.output.scales.dtype
         device = self.output.weight.device
         if dtype != torch.bfloat16:
             raise NotImplementedError(f"the HIP kernels compute in bfloat16 storage; model dtype is {dtype}")
@@ -121,7 +124,7 @@ class GPTBase(nn.Module):
         ws = self._ws.get(key)
         if ws is None:
             w = self.output.weight
-            ws = Workspace(self.config, B, S, self._fused_width(), w.device, w.dtype, self.max_seq_length,
+            ws = Workspace(self.config, B, S, self._fused_width(), w.device, self.norm.weight.dtype, self.max_seq_length,
                            not self.last_logits_only)
             if S > 1:  # keep at most one prefill-sized workspace alive
                 for k in [k for k in self._ws if k[1] > 1]:
@@ -146,10 +149,10 @@ class GPTBase(nn.Module):
             xl = last(ws.x)
             xn = torch.empty_like(xl)
             _hip.add_rmsnorm(xl, last(final_d1), last(final_d2), self.norm.weight, None, xn, cfg.norm_eps)
-            _hip.linear(xn, self.output.weight, ws.logits.view(B, -1))
+            _hip.module_linear(xn, self.output, ws.logits.view(B, -1))
         else:
             _hip.add_rmsnorm(ws.x, final_d1, final_d2, self.norm.weight, None, ws.xn, cfg.norm_eps)
-            _hip.linear(ws.xn, self.output.weight, ws.logits.view(B * S, -1))
+            _hip.module_linear(ws.xn, self.output, ws.logits.view(B * S, -1))
         return ws.logits
 
     def _run_layers(self, ws: Workspace, pos: Tensor):
@@ -158,24 +161,24 @@ class GPTBase(nn.Module):
         raise NotImplementedError
 
     # -- shared pieces of the block schedules -----------------------------------------------------
-    def _attention(self, ws: Workspace, blk, pos: Tensor, wqkv: Tensor, out: Tensor):
+    def _attention(self, ws: Workspace, blk, pos: Tensor, wqkv: nn.Module, out: Tensor):
         """ws.xn -> fused projection -> RoPE + cache write -> attention -> wo -> out (partial sum)."""
         cfg = self.config
         B, S = ws.B, ws.S
         Hq, Hkv, hd = cfg.n_head_local, cfg.n_kv_local, cfg.head_dim
         kc, vc = blk.attention.kv_cache.k_cache, blk.attention.kv_cache.v_cache
-        _hip.linear(ws.xn, wqkv, ws.qkv)
+        _hip.module_linear(ws.xn, wqkv, ws.qkv)
         _hip.rope_kv_write(ws.qkv, self.freqs_cis, False, pos, kc, vc, B, S, Hq, Hkv, hd)
         if S == 1:
             _hip.attn_decode(ws.qkv, kc, vc, pos, ws.y, ws.scratch, B, Hq, Hkv, hd)
         else:
             _hip.attn_prefill(ws.qkv, kc, vc, pos, ws.y, B, S, Hq, Hkv, hd)
-        _hip.linear(ws.y, blk.attention.wo.weight, out)
+        _hip.module_linear(ws.y, blk.attention.wo, out)
 
     def _mlp(self, ws: Workspace, blk, out: Tensor):
         ff = blk.feed_forward
-        _hip.linear(ws.xn, ff.w1.weight, ws.h)
-        _hip.linear_swiglu(ws.h, ff.w2.weight, out, ws.act)
+        _hip.module_linear(ws.xn, ff.w1, ws.h)
+        _hip.module_linear_swiglu(ws.h, ff.w2, out, ws.act)
 
     # -- greedy decoding helper ---------------------------------------------------------------------
     def greedy_next(self, logits: Tensor) -> Tensor:

@@ -34,6 +34,9 @@ class ModelArgs:
     # desync family (gpt_desync_TP.py:44-45)
     reduce_pattern: Optional[List[Dict[str, bool]]] = None
     force_disable_last_all_reduce: bool = False
+    # ladder family: the layers that run the ladder schedule (None: all of them, as gpt_ladder_TP.py does; a list
+    # is the partial-ladder wiring of hf_modeling_utils/modeling_llama_ladder.py:889-948: the others are dense)
+    ladder_layers: Optional[List[int]] = None
     # rank shard: None -> the process-wide virtual setting of gpt_fast.tp
     tp_world_size: Optional[int] = None
     tp_rank: Optional[int] = None
@@ -55,6 +58,13 @@ class ModelArgs:
         assert self.intermediate_size % tp == 0
         if self.reduce_pattern is None:
             self.reduce_pattern = [{"attention": False, "mlp": True} for _ in range(self.n_layer)]
+        if self.ladder_layers is not None:
+            assert all(0 <= i < self.n_layer for i in self.ladder_layers)
+            if sorted(self.ladder_layers) == list(range(self.n_layer)):
+                self.ladder_layers = None
+
+    def is_ladder_layer(self, i: int) -> bool:
+        return self.ladder_layers is None or i in self.ladder_layers
 
     # per-rank sizes
     @property

@@ -50,14 +50,14 @@ class GPTDense(GPTBase):
         for blk in self.layers:
             if blk.keeps_residual:
                 _hip.add_rmsnorm(ws.x, pending, None, blk.attention_norm.weight, ws.x, ws.xn, eps)
-                self._attention(ws, blk, pos, blk.attention.wqkv.weight, ws.a)
+                self._attention(ws, blk, pos, blk.attention.wqkv, ws.a)
                 _hip.add_rmsnorm(ws.x, ws.a, None, blk.ffn_norm.weight, ws.x, ws.xn, eps)
                 self._mlp(ws, blk, ws.m)
                 pending = ws.m
             else:  # the stream is replaced by the module output
                 src = ws.x if pending is None else pending
                 _hip.add_rmsnorm(src, None, None, blk.attention_norm.weight, None, ws.xn, eps)
-                self._attention(ws, blk, pos, blk.attention.wqkv.weight, ws.a)
+                self._attention(ws, blk, pos, blk.attention.wqkv, ws.a)
                 _hip.add_rmsnorm(ws.a, None, None, blk.ffn_norm.weight, None, ws.xn, eps)
                 self._mlp(ws, blk, ws.m)
                 pending = ws.m

@@ -61,7 +61,7 @@ class GPTDesync(GPTBase):
         tp = float(self.config.tp_world_size)
         for blk in self.layers:
             _hip.add_rmsnorm(ws.x, None, None, blk.attention_norm.weight, None, ws.xn, eps)
-            self._attention(ws, blk, pos, blk.attention.wqkv.weight, ws.a)
+            self._attention(ws, blk, pos, blk.attention.wqkv, ws.a)
             _hip.add(ws.a, ws.x, ws.x, tp if blk.do_attention_all_reduce else 1.0)
             _hip.add_rmsnorm(ws.x, None, None, blk.ffn_norm.weight, None, ws.xn, eps)
             self._mlp(ws, blk, ws.m)

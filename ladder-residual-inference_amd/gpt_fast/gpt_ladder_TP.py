@@ -76,7 +76,10 @@ class GPTLadder(GPTBase):
         if st is None:
             st = self._fused = {}
         if B not in st:
-            st[B] = _hip.FusedLadderStep(self, B) if B <= 2 else None
+            # the one-kernel step implements the all-ladder schedule only, on bf16 weights
+            ok = B <= 2 and self.config.ladder_layers is None and self.output.weight.dtype == torch.bfloat16 and \
+                all(p.dtype == torch.bfloat16 for p in self.layers[0].state_dict().values() if p.dim() == 2)
+            st[B] = _hip.FusedLadderStep(self, B) if ok else None
             if st[B] is not None and not st[B].supported:
                 st[B] = None
         return st[B]
@@ -112,13 +115,25 @@ class GPTLadder(GPTBase):
         return super().greedy_next(logits)
 
     def _run_layers(self, ws: Workspace, pos: Tensor):
-        eps = self.config.norm_eps
+        cfg = self.config
+        eps = cfg.norm_eps
         pending_a = pending_m = None  # the reference starts from zero tensors; adding zero is the identity
-        for blk in self.layers:
-            _hip.add_rmsnorm(ws.x, pending_a, None, blk.attention_norm.weight, ws.x, ws.xn, eps)
-            self._attention(ws, blk, pos, blk.attention.wqkv.weight, ws.a)
-            pending_a = ws.a
-            _hip.add_rmsnorm(ws.x, pending_m, None, blk.ffn_norm.weight, ws.x, ws.xn, eps)
-            self._mlp(ws, blk, ws.m)
-            pending_m = ws.m
+        for i, blk in enumerate(self.layers):
+            if cfg.is_ladder_layer(i):
+                _hip.add_rmsnorm(ws.x, pending_a, None, blk.attention_norm.weight, ws.x, ws.xn, eps)
+                self._attention(ws, blk, pos, blk.attention.wqkv, ws.a)
+                pending_a = ws.a
+                _hip.add_rmsnorm(ws.x, pending_m, None, blk.ffn_norm.weight, ws.x, ws.xn, eps)
+                self._mlp(ws, blk, ws.m)
+                pending_m = ws.m
+            else:
+                # a dense layer of a partial-ladder model (modeling_llama_ladder.py:614-637): it sees everything
+                # produced so far, adds its attention output at once, and leaves its MLP output pending -- the
+                # next layer adds it first (dense) or after its attention (ladder: "prev_attn_output" is this
+                # layer's state before the MLP output, :644-658)
+                _hip.add_rmsnorm(ws.x, pending_a, pending_m, blk.attention_norm.weight, ws.x, ws.xn, eps)
+                self._attention(ws, blk, pos, blk.attention.wqkv, ws.a)
+                _hip.add_rmsnorm(ws.x, ws.a, None, blk.ffn_norm.weight, ws.x, ws.xn, eps)
+                self._mlp(ws, blk, ws.m)
+                pending_a, pending_m = None, ws.m
         return pending_a, pending_m

@@ -49,8 +49,8 @@ class GPTParallel(GPTBase):
         for blk in self.layers:
             att = blk.attention
             _hip.add_rmsnorm(ws.x, None, None, blk.attention_norm.weight, None, ws.xn, cfg.norm_eps)
-            self._attention(ws, blk, pos, att.wqkv1.weight, ws.a)   # ws.qkv holds [q | k | v | u | g]
-            _hip.linear_swiglu(ws.qkv[:, nqkv:], att.w2.weight, ws.m, ws.act)
+            self._attention(ws, blk, pos, att.wqkv1, ws.a)   # ws.qkv holds [q | k | v | u | g]
+            _hip.module_linear_swiglu(ws.qkv[:, nqkv:], att.w2, ws.m, ws.act)
             _hip.add(ws.m, ws.a, ws.m)                               # w2(...) + wo(...)
             if blk.keeps_residual:
                 _hip.add(ws.m, ws.x, ws.x)                           # y + x

@@ -129,8 +129,8 @@ class FeedForward(nn.Module):
     def forward(self, x: Tensor) -> Tensor:
         x = x.contiguous()
         lead = x.shape[:-1]
-        h = _hip.linear(x, self.w1.weight, x.new_empty(*lead, self.w1.out_features))
-        return _hip.linear_swiglu(h, self.w2.weight, x.new_empty(*lead, self.w2.out_features))
+        h = _hip.module_linear(x, self.w1, x.new_empty(*lead, self.w1.out_features))
+        return _hip.module_linear_swiglu(h, self.w2, x.new_empty(*lead, self.w2.out_features))
 
 
 class _AttentionCore(nn.Module):
@@ -196,9 +196,9 @@ class Attention(_AttentionCore):
     def forward(self, x: Tensor, freqs_cis: Tensor, mask: Tensor, input_pos: Optional[Tensor] = None) -> Tensor:
         bsz, seqlen, _ = x.shape
         x = x.contiguous()
-        qkv = _hip.linear(x, self.wqkv.weight, x.new_empty(bsz, seqlen, self.wqkv.out_features))
+        qkv = _hip.module_linear(x, self.wqkv, x.new_empty(bsz, seqlen, self.wqkv.out_features))
         y = self._attend(qkv, bsz, seqlen, freqs_cis, input_pos)
-        return _hip.linear(y, self.wo.weight, x.new_empty(bsz, seqlen, self.wo.out_features))
+        return _hip.module_linear(y, self.wo, x.new_empty(bsz, seqlen, self.wo.out_features))
 
 
 class FuseAttentionMLP(_AttentionCore):
@@ -221,8 +221,8 @@ class FuseAttentionMLP(_AttentionCore):
         bsz, seqlen, _ = x.shape
         x = x.contiguous()
         nqkv = (self.n_head + 2 * self.n_local_heads) * self.head_dim
-        fused = _hip.linear(x, self.wqkv1.weight, x.new_empty(bsz, seqlen, self.wqkv1.out_features))
+        fused = _hip.module_linear(x, self.wqkv1, x.new_empty(bsz, seqlen, self.wqkv1.out_features))
         y = self._attend(fused, bsz, seqlen, freqs_cis, input_pos)
-        a = _hip.linear(y, self.wo.weight, x.new_empty(bsz, seqlen, self.wo.out_features))
-        m = _hip.linear_swiglu(fused[..., nqkv:], self.w2.weight, x.new_empty(bsz, seqlen, self.w2.out_features))
+        a = _hip.module_linear(y, self.wo, x.new_empty(bsz, seqlen, self.wo.out_features))
+        m = _hip.module_linear_swiglu(fused[..., nqkv:], self.w2, x.new_empty(bsz, seqlen, self.w2.out_features))
         return _hip.add(m, a, m)

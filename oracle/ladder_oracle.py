@@ -21,6 +21,7 @@ torch.distributed and no module state, the maths of
   gpt_fast/utils.py:305-387                    fused attention+MLP of the parallel block
   gpt_fast/utils.py:390-397                    all-reduce  -> identity (partial sums stay local)
   benchmark.py:58-164                          sampling / prefill / decode loop (greedy added)
+  gpt_fast/gpt_ladder_TP.py:233-237            hook for weight-only quantised linears (fp8 form restated)
 
 Every tensor is rounded to the model dtype exactly where the eager reference
 rounds it: after each add, after the normalisation and again after the gain,
@@ -72,6 +73,9 @@ class OracleConfig:
     # desync only (gpt_desync_TP.py:44-45, 59-60)
     reduce_pattern: Optional[List[Dict[str, bool]]] = None
     force_disable_last_all_reduce: bool = False
+    # layers that run the ladder schedule (None: all); the others are dense -- the partial-ladder wiring of
+    # hf_modeling_utils/modeling_llama_ladder.py:889-948
+    ladder_layers: Optional[List[int]] = None
     # rank shard: sizes are divided by this; no collective is issued
     tp_world_size: int = 1
     # lm_head rows kept by this rank (None: full vocab, as the reference does)
@@ -170,6 +174,51 @@ def rms_norm(x: Tensor, weight: Tensor, eps: float) -> Tensor:
     xf = x.float()
     n = (xf * torch.rsqrt(torch.mean(xf * xf, dim=-1, keepdim=True) + eps)).type_as(x)
     return n * weight
+
+
+# --- weight-only fp8 linears.  The reference only leaves the hook of gpt-fast's weight-only quantisation
+# (gpt_ladder_TP.py:233-237: a quantised nn.Linear replacement keeps `weight` in the narrow type and a
+# per-output-row `scales` in the model dtype); the arithmetic restated here is that scheme's,
+#     y = F.linear(x, weight.to(x.dtype)) * scales,
+# with e4m3 weights.  No reference file carries the quantiser or the quantised forward, so parity at
+# this boundary is "parity unpinned"; the functions are pinned by closed forms (tests/test_oracle_ops.py).
+FP8_MAX = 448.0  # largest finite float8_e4m3fn
+
+
+def quantize_fp8_rowwise(w: Tensor, scale_dtype=torch.bfloat16) -> Tuple[Tensor, Tensor]:
+    """w [N, K] -> (float8_e4m3fn [N, K], scales [N] in scale_dtype): row n is stored as w[n] / scales[n]
+    with scales[n] = max|w[n]| / 448 rounded to scale_dtype (rows of zeros get scale 1)."""
+    amax = w.float().abs().amax(dim=1)
+    scales = torch.where(amax > 0, amax / FP8_MAX, torch.ones_like(amax)).to(scale_dtype)
+    q = (w.float() / scales.float()[:, None]).clamp(-FP8_MAX, FP8_MAX).to(torch.float8_e4m3fn)
+    return q, scales
+
+
+def linear_fp8(x: Tensor, w8: Tensor, scales: Tensor) -> Tensor:
+    """F.linear(x, w8.to(x.dtype)) * scales: the e4m3 -> bf16 conversion is exact, the product is rounded to
+    x.dtype by the matmul and once more after the scaling."""
+    return F.linear(x, w8.to(x.dtype)) * scales.to(x.dtype)
+
+
+def linear(P: Dict[str, Tensor], name: str, x: Tensor) -> Tensor:
+    """nn.Linear without bias on parameter `name` of P; the weight-only fp8 form if P holds
+    `<module>.scales` beside `<module>.weight`."""
+    scales = P.get(name[: -len("weight")] + "scales")
+    if scales is not None:
+        return linear_fp8(x, P[name], scales)
+    return F.linear(x, P[name])
+
+
+def quantize_params_fp8(P: Dict[str, Tensor]) -> Dict[str, Tensor]:
+    """Every projection (wqkv, wqkv1, wo, w1, w2, output) of a parameter dict in the weight-only fp8 form;
+    norm gains and the embedding table stay as they are."""
+    out = {}
+    for name, w in P.items():
+        if w.dim() == 2 and name != "tok_embeddings.weight":
+            out[name], out[name[: -len("weight")] + "scales"] = quantize_fp8_rowwise(w, w.dtype)
+        else:
+            out[name] = w
+    return out
 
 
 def rope_scaled_freqs(freqs: Tensor, rope_scaling: dict) -> Tensor:
@@ -281,16 +330,16 @@ def attention(cfg: OracleConfig, P: Dict[str, Tensor], layer: int, x: Tensor, ca
     """utils.py:187-260 (non-flash).  wqkv rows are [q_local; k_local; v_local]."""
     p = f"layers.{layer}.attention."
     hd = cfg.head_dim
-    q, k, v = F.linear(x, P[p + "wqkv.weight"]).split([cfg.hq * hd, cfg.hkv * hd, cfg.hkv * hd], dim=-1)
+    q, k, v = linear(P, p + "wqkv.weight", x).split([cfg.hq * hd, cfg.hkv * hd, cfg.hkv * hd], dim=-1)
     y = _attn_core(cfg, q, k, v, layer, caches, freqs_cis, mask, input_pos)
-    return F.linear(y, P[p + "wo.weight"])  # row-parallel: a partial sum
+    return linear(P, p + "wo.weight", y)  # row-parallel: a partial sum
 
 
 def feed_forward(cfg: OracleConfig, P: Dict[str, Tensor], layer: int, x: Tensor) -> Tensor:
     """utils.py:145-149.  w1 rows are [up; gate]: u is the FIRST half, g the second."""
     p = f"layers.{layer}.feed_forward."
-    u, g = F.linear(x, P[p + "w1.weight"]).chunk(2, dim=-1)
-    return F.linear(F.silu(g) * u, P[p + "w2.weight"])  # row-parallel: a partial sum
+    u, g = linear(P, p + "w1.weight", x).chunk(2, dim=-1)
+    return linear(P, p + "w2.weight", F.silu(g) * u)  # row-parallel: a partial sum
 
 
 def fused_attention_mlp(cfg: OracleConfig, P: Dict[str, Tensor], layer: int, x: Tensor, caches: OracleCaches,
@@ -298,11 +347,11 @@ def fused_attention_mlp(cfg: OracleConfig, P: Dict[str, Tensor], layer: int, x: 
     """utils.py:305-387.  wqkv1 rows are [q; k; v; u; g]; result = w2(silu(g) u) + wo(y)."""
     p = f"layers.{layer}.attention."
     hd = cfg.head_dim
-    q, k, v, u, g = F.linear(x, P[p + "wqkv1.weight"]).split(
+    q, k, v, u, g = linear(P, p + "wqkv1.weight", x).split(
         [cfg.hq * hd, cfg.hkv * hd, cfg.hkv * hd, cfg.ffn, cfg.ffn], dim=-1)
     y = _attn_core(cfg, q, k, v, layer, caches, freqs_cis, mask, input_pos)
-    y = F.linear(y, P[p + "wo.weight"])
-    return F.linear(F.silu(g) * u, P[p + "w2.weight"]) + y
+    y = linear(P, p + "wo.weight", y)
+    return linear(P, p + "w2.weight", F.silu(g) * u) + y
 
 
 # --------------------------------------------------------------------------------------
@@ -328,7 +377,7 @@ def _prologue(P, caches, idx, input_pos):
 
 
 def _epilogue(cfg, P, x):
-    return F.linear(rms_norm(x, P["norm.weight"], cfg.norm_eps), P["output.weight"])  # :282-283
+    return linear(P, "output.weight", rms_norm(x, P["norm.weight"], cfg.norm_eps))  # :282-283
 
 
 def forward_ladder(cfg: OracleConfig, P: Dict[str, Tensor], caches: OracleCaches, idx: Tensor,
@@ -338,7 +387,18 @@ def forward_ladder(cfg: OracleConfig, P: Dict[str, Tensor], caches: OracleCaches
     pa = torch.zeros_like(x)
     pm = torch.zeros_like(x)
     for i in range(cfg.n_layer):
-        pa, pm, x = ladder_block(cfg, P, i, pa, pm, x, caches, freqs_cis, mask, input_pos)
+        if cfg.ladder_layers is None or i in cfg.ladder_layers:
+            pa, pm, x = ladder_block(cfg, P, i, pa, pm, x, caches, freqs_cis, mask, input_pos)
+        else:
+            # dense layer of a partial-ladder model (modeling_llama_ladder.py:614-637, 889-948), in the
+            # pending-sum form: it reads the full sum, adds its attention output at once and leaves its MLP
+            # output pending (a following ladder layer's attention must not see it, :644)
+            p = f"layers.{i}."
+            x = x + pa + pm
+            x = x + attention(cfg, P, i, rms_norm(x, P[p + "attention_norm.weight"], cfg.norm_eps),
+                              caches, freqs_cis, mask, input_pos)
+            pm = feed_forward(cfg, P, i, rms_norm(x, P[p + "ffn_norm.weight"], cfg.norm_eps))
+            pa = torch.zeros_like(x)
     x = x + pa + pm                                                                # :280
     return _epilogue(cfg, P, x)
 
@@ -435,7 +495,7 @@ def generate(cfg: OracleConfig, P: Dict[str, Tensor], prompt: Tensor, max_new_to
 
     fwd = FORWARD[family]
     dev = prompt.device
-    dtype = P["output.weight"].dtype
+    dtype = P["output.scales"].dtype if "output.scales" in P else P["output.weight"].dtype   # gpt_ladder_TP.py:232-237
     T = prompt.numel()
     if caches is None:
         caches = setup_caches(cfg, batch_size, min(T + max_new_tokens, cfg.block_size), dtype, dev)

@@ -69,6 +69,7 @@ def oracle_cfg(c) -> O.OracleConfig:
                           dim=c.dim, intermediate_size=c.intermediate_size, n_local_heads=c.n_local_heads,
                           rope_base=c.rope_base, norm_eps=c.norm_eps, rope_scaling=c.rope_scaling,
                           reduce_pattern=c.reduce_pattern, force_disable_last_all_reduce=c.force_disable_last_all_reduce,
+                          ladder_layers=c.ladder_layers,
                           tp_world_size=c.tp_world_size, vocab_shard=c.output_rows if c.shard_vocab else None)
 
 
@@ -467,6 +468,34 @@ def test_sample_goes_through_the_device_sampler_and_matches_the_oracle():
     # greedy flag: the device argmax
     tok_g, none = bm.sample(logits, greedy=True, model=model)
     assert none is None and torch.equal(tok_g, torch.argmax(logits[:, -1], -1, keepdim=True).to(torch.int32))
+
+
+# ---------------------------------------------------------------------------------------------------
+# weight-only fp8 decode
+# ---------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("family", ["ladder", "dense", "parallel"])
+def test_tiny_models_with_fp8_weights(family):
+    from gpt_fast.quantize import quantize_model_fp8
+
+    model = quantize_model_fp8(build(family, **dict(TINY, dim=256, intermediate_size=512)))
+    assert model.output.weight.dtype == torch.float8_e4m3fn and "layers.0.attention.wo.scales" in model.state_dict()
+    stats = run_parity(model, family, B=2, T=20, new=10)
+    print(family, stats)
+    check(stats)
+    assert not stats["fused_step_used"]
+
+
+@pytest.mark.parametrize("B", [1, 8])
+def test_ladder_70b_tp8_shard_shape_with_fp8_weights(B):
+    """The 70B rank shard's matrices (12 layers) in the weight-only fp8 form: prefill (expanded weights, matrix-core
+    GEMM) and decode (fp8 GEMV) against the oracle on the same fp8 weights and scales."""
+    from gpt_fast.quantize import quantize_model_fp8
+
+    model = quantize_model_fp8(build("ladder", **shape_kw("ladder-70b-tp8", 12)))
+    stats = run_parity(model, "ladder", B=B, T=512, new=24)
+    report(f"fp8 weights, cfg3 shape, 12 layers, B={B}", stats)
+    check(stats)
 
 
 # ---------------------------------------------------------------------------------------------------

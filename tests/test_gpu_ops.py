@@ -246,6 +246,46 @@ def test_rope_kv_write_exact(hip, hd, Hq, Hkv, gathered):
     assert torch.equal(work[..., Hq * hd:], torch.cat([k, v], -1))   # k and v columns are left as they were
 
 
+# ------------------------------------------------------------------------------------ weight-only fp8 linear
+
+def test_linear_fp8_decodes_every_e4m3_value_exactly(hip):
+    """All 254 finite byte patterns of float8_e4m3fn (normals, denormals, both zeros) through the kernel's
+    conversion: with one-hot inputs and unit scales the output IS the stored value."""
+    codes = torch.arange(256, dtype=torch.uint8, device=DEV)
+    codes[0x7F] = 0          # the two NaN patterns are replaced
+    codes[0xFF] = 0x80
+    w8 = codes.view(torch.float8_e4m3fn).view(16, 16).contiguous()
+    scales = torch.ones(16, dtype=BF, device=DEV)
+    want = w8.to(torch.float32).T.contiguous()      # y[m, n] = w8[n, m]
+    for m0 in (0, 8):
+        x = torch.eye(16, dtype=BF, device=DEV)[m0:m0 + 8].contiguous()
+        y = torch.empty(8, 16, dtype=BF, device=DEV)
+        hip.linear_fp8(x, w8, scales, y)
+        assert torch.equal(y.float(), want[m0:m0 + 8])
+    assert want.abs().max().item() == 448.0 and (want.abs()[want != 0].min().item() == 2.0 ** -9)
+
+
+@pytest.mark.parametrize("N,K", [(1280, 8192), (8192, 1024), (7168, 8192), (8192, 3584), (16032, 8192), (3072, 2048),
+                                 (1001, 528), (24, 64)])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 16, 300])
+def test_linear_fp8(hip, M, N, K):
+    """Decode (M <= 8: fp8 weights streamed once) and prefill (M > 8: expanded to bf16 in scratch + matrix-core
+    GEMM + column scaling) against the oracle's F.linear(x, w8.to(bf16)) * scales."""
+    if M == 300 and N * K > 30e6:
+        M = 64
+    x = rnd(M, K, seed=40)
+    w8, scales = O.quantize_fp8_rowwise(rnd(N, K, seed=41, scale=0.02, dtype=torch.float32), BF)
+    y = torch.empty(M, N, dtype=BF, device=DEV)
+    hip.linear_fp8(x, w8, scales, y)
+    want = O.linear_fp8(x, w8, scales)
+    # two roundings (the sum, then the scaled sum): a one-step difference in the first can survive as one or,
+    # through double rounding, two steps of the result
+    assert_close_ulp(y, want, max_ulp=2, max_frac=0.06, what=f"fp8 linear M={M} N={N} K={K}")
+    exact = ((x.double() @ w8.double().T) * scales.double()).to(BF)
+    # (the single rounding of the exact product differs from the two roundings of the scheme at about a quarter of the elements, by one step)
+    assert_close_ulp(y, exact, max_ulp=2, max_frac=0.4, what="fp8 linear vs fp64")
+
+
 def test_rope_kv_write_position_out_of_range_sets_the_error_word(hip):
     """Positions beyond the cache or the RoPE table: the row is left alone, nothing lands in the cache and the
     per-device error word becomes LR_DEV_POS_RANGE (the reference raises an index error, utils.py:55)."""

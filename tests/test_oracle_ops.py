@@ -332,3 +332,55 @@ def test_greedy_first_maximum_on_ties_int32():
     t = O.greedy(lg)
     assert t.dtype == torch.int32 and t.shape == (2, 1) and t.flatten().tolist() == [4, 2]
     assert O.greedy(lg.to(torch.bfloat16)).flatten().tolist() == [4, 2]
+
+
+# ------------------------------------------------------------------------------------ weight-only fp8
+
+def test_fp8_quantiser_closed_forms():
+    """quantize_fp8_rowwise / linear_fp8 (the weight-only scheme behind gpt_ladder_TP.py:233-237) against what
+    the definition fixes: the row maximum lands on +-448, every element is within half an e4m3 step of the
+    scaled weight, a row of zeros stays zero, and the product equals the fp64 product of the de-quantised
+    matrix up to the two stated bf16 roundings."""
+    g = torch.Generator().manual_seed(0)
+    w = torch.randn(33, 64, generator=g) * 0.02
+    w[5] = 0.0
+    w[7, 3] = 0.5        # a row dominated by one element: the rest falls into the denormal range of e4m3
+    q, s = O.quantize_fp8_rowwise(w)
+    assert q.dtype == torch.float8_e4m3fn and s.dtype == torch.bfloat16 and s.shape == (33,)
+    qf, sf = q.float(), s.float()
+    amax = w.abs().amax(1)
+    live = amax > 0
+    assert torch.equal(qf.abs().amax(1)[live], torch.full((32,), 448.0))
+    assert ((sf[live] - amax[live] / 448).abs() <= 2.0 ** -8 * sf[live]).all() and sf[5] == 1.0 and (qf[5] == 0).all()
+    # e4m3: 3 mantissa bits -> relative half-step 2^-4 for normal values, absolute half-step 2^-10 below 2^-6
+    target = w / sf[:, None]
+    err = (qf - target.clamp(-448, 448)).abs()
+    assert (err <= torch.maximum(target.abs() * 2.0 ** -4, torch.tensor(2.0 ** -10))).all()
+    # a wrong-way division (w * scale) or a dropped clamp would break the lines above; now the product
+    x = (torch.randn(5, 64, generator=g)).to(torch.bfloat16)
+    y = O.linear_fp8(x, q, s)
+    exact = (x.double() @ qf.double().T) * sf.double()
+    assert y.dtype == torch.bfloat16
+    assert ((y.double() - exact).abs() <= 2.0 ** -7 * exact.abs() + 1e-30).all()
+    assert (y[:, 5] == 0).all()
+    # and it is NOT the plain linear on the original weights (negative control), though close to it
+    plain = torch.nn.functional.linear(x.float(), w)
+    assert 1e-3 < ((y.float() - plain).abs().max() / plain.abs().max()).item() < 0.2
+
+
+def test_fp8_parameter_dict_and_dispatch():
+    cfg = O.OracleConfig(block_size=16, vocab_size=64, n_layer=1, n_head=2, dim=32, intermediate_size=48)
+    P = O.init_params(cfg, seed=0, dtype=torch.bfloat16, std=0.1)
+    Q = O.quantize_params_fp8(P)
+    assert Q["tok_embeddings.weight"] is P["tok_embeddings.weight"] and Q["norm.weight"] is P["norm.weight"]
+    for n in ("layers.0.attention.wqkv", "layers.0.attention.wo", "layers.0.feed_forward.w1", "layers.0.feed_forward.w2",
+              "output"):
+        assert Q[n + ".weight"].dtype == torch.float8_e4m3fn and Q[n + ".scales"].shape == (P[n + ".weight"].shape[0],)
+    x = torch.randn(3, 32).to(torch.bfloat16)
+    assert torch.equal(O.linear(Q, "output.weight", x), O.linear_fp8(x, Q["output.weight"], Q["output.scales"]))
+    assert torch.equal(O.linear(P, "output.weight", x), torch.nn.functional.linear(x, P["output.weight"]))
+    # the quantised model's logits stay close to the unquantised ones (the scheme is a small perturbation)
+    idx = torch.randint(0, 64, (1, 5))
+    lp = O.forward_ladder(cfg, P, O.setup_caches(cfg, 1, 16, torch.bfloat16), idx, torch.arange(5)).float()
+    lq = O.forward_ladder(cfg, Q, O.setup_caches(cfg, 1, 16, torch.bfloat16), idx, torch.arange(5)).float()
+    assert 0 < ((lp - lq).abs().max() / lp.abs().max()).item() < 0.25
