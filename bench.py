@@ -24,7 +24,16 @@ Prints ONE JSON line.  `value` = decoded tokens per second (whole job = the one 
                token hand-over): algorithmic bytes per step / measured step time.
 `cpu_baseline`: the oracle (a PyTorch-CPU restatement of the reference; the reference itself cannot
                run without CUDA + NCCL) timed on this machine's host cores on the reference's
-               CPU-sized case: Ladder-1B fp32, batch 1, 128-token prompt, greedy decode."""
+               CPU-sized case: Ladder-1B fp32, batch 1, 128-token prompt, greedy decode.  `cores` =
+               threads used (the process's CPU share: OMP_NUM_THREADS when set, else every core),
+               `host_cpus` = os.cpu_count().
+Measured in the same run and reported as extra keys (not the headline; --no-extras skips them):
+`batched`     : the same rank shard at batch 8 and 64 (per-op kernels, hipGraph replay): ms per step,
+               tok/s, algorithmic GB/s and its fraction of 8 TB/s.
+`fp8`         : the same shard with weight-only e4m3 projections at batch 1 (per-op kernels): ms per
+               step and the fraction of 8 TB/s on ITS algorithmic bytes (one byte per weight + scales).
+`prefill`     : Ladder-8B, batch 32 x 2048 prompt tokens, causal prefill with last-position logits:
+               seconds, algorithmic TFLOP/s and the fraction of 2.5 PFLOP/s (dense bf16 MFMA peak)."""
 import argparse
 import json
 import os
@@ -36,9 +45,10 @@ sys.path.insert(0, os.path.join(ROOT, "ladder-residual-inference_amd"))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes one k_ladder_step launch moves on the headline workload, from the rocprofv3 counter runs
-# summarised under profiles/ (None until measured).
-TRAFFIC_BYTES_PER_LAUNCH = 17.692e9  # B=1, prompt 2048; 1.013 x algorithmic
+MFMA_PEAK_TFLOPS = 2500.0   # dense bf16
+# HBM bytes one launch of the dominant kernel moves, per workload (model, batch, prompt), from the rocprofv3
+# FETCH_SIZE / WRITE_SIZE counter runs summarised under profiles/; workloads without a counter run report null.
+TRAFFIC_BYTES_PER_LAUNCH = {("gpt_ladder:ladder-70b-tp8", 1, 2048): 17.65e9}   # 1.011 x algorithmic
 
 
 def cpu_baseline(new_tokens=32, repeats=2):
@@ -47,7 +57,10 @@ def cpu_baseline(new_tokens=32, repeats=2):
 
     from oracle import ladder_oracle as O
 
-    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    host_cpus = os.cpu_count() or 1
+    # the process may own only a share of the host (the harness exports it as OMP_NUM_THREADS): more threads than
+    # that only fight each other
+    cores = min(host_cpus, int(os.environ.get("OMP_NUM_THREADS", host_cpus)))
     torch.set_num_threads(cores)
     cfg = O.OracleConfig(block_size=2048, vocab_size=128256, n_layer=16, n_head=32, n_local_heads=8, dim=2048,
                          intermediate_size=8192, rope_base=500000)
@@ -64,10 +77,105 @@ def cpu_baseline(new_tokens=32, repeats=2):
         dec.append(tm["decode_latency"] / (new_tokens - 1))
         pre.append(tm["prefill_latency"])
     ms = 1e3 * sum(dec) / len(dec)
-    return {"value": round(1e3 / ms, 3), "unit": "tok/s", "cores": cores, "kind": "port",
+    return {"value": round(1e3 / ms, 3), "unit": "tok/s", "cores": cores, "host_cpus": host_cpus, "kind": "port",
             "ms_per_token": round(ms, 3), "prefill_s": round(sum(pre) / len(pre), 3),
             "sample": f"oracle (PyTorch CPU fp32) on Ladder-1B (dim 2048, 16 layers, 32q/8kv, FFN 8192, vocab 128256), "
                       f"B=1, prompt 128, greedy decode of {new_tokens} tokens, {repeats} runs"}
+
+
+def decode_run(bm, model, prompt, B, T, K, W):
+    """Prefill the prompt at batch B, capture the decode step, run W untimed + K timed steps from position T.
+    Returns (ms per step, first token tensor, DecodeGraph)."""
+    import torch
+
+    new = max(K, W) + 1
+    model.max_seq_length = -1            # new caches for this batch size
+    model.setup_caches(B, T + max(new, 128))
+    rows = prompt.view(1, -1).repeat(B, 1)
+    first = bm.prefill(model, rows, torch.arange(T, device=prompt.device, dtype=torch.int32), greedy=True).clone()
+    dg = bm.get_cuda_graphs_for_decode(model, prompt, B, new, first, greedy=True)
+    dg.reset(first)
+    for _ in range(W):
+        dg.replay()
+    dg.reset(first)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(K):
+        dg.replay()
+    torch.cuda.synchronize()
+    ms = 1e3 * (time.perf_counter() - t0) / K
+    model.check_device_errors()
+    return ms, first, dg
+
+
+def extra_batched(bm, model, prompt, T, batches=(8, 64), K=32, W=5):
+    """The headline shard at the other batch sizes of the benchmark set (per-op kernels)."""
+    cfg = model.config
+    out = []
+    for B in batches:
+        ms, _, dg = decode_run(bm, model, prompt, B, T, K, W)
+        nbytes = sum(bm.decode_bytes_per_step(cfg, B, T + i) for i in range(K)) / K
+        gbps = nbytes / (ms * 1e-3) / 1e9
+        out.append({"batch": B, "ms_per_step": round(ms, 4), "tok_per_s": round(B * 1e3 / ms, 1),
+                    "bytes_per_step": int(nbytes), "achieved_GBps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4),
+                    "steps": K})
+        del dg
+    return out
+
+
+def fp8_bytes_per_step(cfg, B, pos):
+    """decode_bytes_per_step with one byte per projection weight plus a bf16 scale per output row."""
+    D, L, hd = cfg.dim, cfg.n_layer, cfg.head_dim
+    Hq, Hkv, I, V = cfg.n_head_local, cfg.n_kv_local, cfg.ffn_local, cfg.output_rows
+    nqkv = (Hq + 2 * Hkv) * hd
+    w = L * (D * nqkv + D * Hq * hd + D * 2 * I + I * D) + V * D                   # one byte each
+    scales = 2 * (L * (nqkv + D + 2 * I + D) + V)
+    gains = 2 * (L * 2 * D + D)
+    kv = 2 * (L * B * 2 * Hkv * hd * (pos + 1) + L * B * 2 * Hkv * hd) + 2 * B * D
+    return w + scales + gains + kv
+
+
+def extra_fp8(bm, model, prompt, T, K=32, W=5):
+    """Weight-only e4m3 projections on the headline shard, batch 1.  Quantises `model` in place (call it last)."""
+    from gpt_fast.quantize import quantize_model_fp8
+
+    quantize_model_fp8(model)
+    ms, _, dg = decode_run(bm, model, prompt, 1, T, K, W)
+    nbytes = sum(fp8_bytes_per_step(model.config, 1, T + i) for i in range(K)) / K
+    gbps = nbytes / (ms * 1e-3) / 1e9
+    return {"batch": 1, "ms_per_step": round(ms, 4), "tok_per_s": round(1e3 / ms, 1), "bytes_per_step": int(nbytes),
+            "achieved_GBps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4), "steps": K,
+            "kernels": "per-op (fp8 GEMV), hipGraph replay"}
+
+
+def extra_prefill(bm, B=32, T=2048, reps=2):
+    """Config 4: Ladder-8B, B x T prompt tokens, causal prefill, logits of the last position."""
+    import torch
+
+    model = bm._load_model("gpt_ladder:ladder-8b", "cuda", torch.bfloat16, seed=0, verbose=False)
+    model.last_logits_only = True
+    c = model.config
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1)
+    rows = torch.randint(0, c.vocab_size, (T,), device="cuda", generator=g).view(1, -1).repeat(B, 1)
+    pos = torch.arange(T, device="cuda", dtype=torch.int32)
+    model.setup_caches(B, T + 8)
+    bm.prefill(model, rows, pos, greedy=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        bm.prefill(model, rows, pos, greedy=True)
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / reps
+    model.check_device_errors()
+    D, L, hd, Hq, Hkv, I, V = c.dim, c.n_layer, c.head_dim, c.n_head_local, c.n_kv_local, c.ffn_local, c.output_rows
+    lin = 2 * B * T * L * (D * (Hq + 2 * Hkv) * hd + D * Hq * hd + 3 * D * I) + 2 * B * V * D
+    att = L * B * Hq * 2 * hd * T * T
+    tf = (lin + att) / sec / 1e12
+    return {"workload": f"gpt_ladder:ladder-8b, batch {B} x {T} prompt tokens, causal prefill, last-position logits",
+            "seconds": round(sec, 4), "flop": int(lin + att), "achieved_TFLOPs": round(tf, 1),
+            "peak_TFLOPs": MFMA_PEAK_TFLOPS, "frac": round(tf / MFMA_PEAK_TFLOPS, 4),
+            "prompt_tok_per_s": round(B * T / sec, 1)}
 
 
 def main():
@@ -79,6 +187,8 @@ def main():
     ap.add_argument("--prompt", type=int, default=2048)
     ap.add_argument("--model", type=str, default="gpt_ladder:ladder-70b-tp8")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the extra keys (other batch sizes, fp8 weights, the prefill-heavy configuration)")
     ap.add_argument("--per-op", action="store_true",
                     help="decode with one kernel per operation (captured in the hipGraph) instead of the persistent "
                          "one-kernel step: the comparison point, not the headline")
@@ -218,7 +328,8 @@ def main():
         "prefill_s": round(prefill_s, 4),
         "roofline": {"bound": "hbm", "kernel": k_name,
                      "achieved": round(k_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(k_gbps / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH if fused else None,
+                     "frac": round(k_gbps / HBM_PEAK_GBPS, 4),
+                     "traffic": TRAFFIC_BYTES_PER_LAUNCH.get((args.model, B, T)) if fused else None,
                      "bytes_per_launch": int(k_bytes), "avg_launch_us": round(k_us, 3),
                      "measured_read_ceiling": round(ceiling_gbps, 1),
                      "frac_of_measured_ceiling": round(k_gbps / ceiling_gbps, 4)},
@@ -226,9 +337,17 @@ def main():
                           "frac": round(step_gbps / HBM_PEAK_GBPS, 4), "bytes_per_step": int(step_bytes)},
         "first_tokens": tokens,
     }
-    if not args.no_cpu_baseline:
-        del dg, model
+    del dg
+    if not args.no_extras and args.model == "gpt_ladder:ladder-70b-tp8" and B == 1:
+        out["batched"] = extra_batched(bm, model, prompt, T)
+        out["fp8"] = extra_fp8(bm, model, prompt, T)
+        del model
         torch.cuda.empty_cache()
+        out["prefill"] = extra_prefill(bm)
+    else:
+        del model
+    torch.cuda.empty_cache()
+    if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out), flush=True)
 

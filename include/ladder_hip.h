@@ -75,6 +75,16 @@ int lr_add(const void* a, const void* b, float b_div, void* out, int64_t n, lr_s
 int lr_add_rmsnorm(const void* resid_in, const void* d1, const void* d2, const void* gain, void* resid_out,
                    void* normed_out, int rows, int dim, float eps, lr_stream_t stream);
 
+/* Both residual updates and both RMSNorms of one ladder block in one launch:
+ *     r1 = bf16(resid_in + d1),  normed1 = norm(r1) * gain1      (gpt_ladder_TP.py:326-337)
+ *     r2 = bf16(r1 + d2),        normed2 = norm(r2) * gain2      (gpt_ladder_TP.py:346-354)
+ *     resid_out = r2
+ * with norm() as in lr_add_rmsnorm.  Legal because the block's MLP input does not contain the block's own
+ * attention output (that is the ladder schedule): attention(normed1) and mlp(normed2) can then run
+ * side by side, e.g. on two streams.  d1 / d2 may be NULL (the first block); resid_out may alias resid_in. */
+int lr_ladder_norms(const void* resid_in, const void* d1, const void* d2, const void* gain1, const void* gain2,
+                    void* resid_out, void* normed1, void* normed2, int rows, int dim, float eps, lr_stream_t stream);
+
 /* y[m, n] = bf16( sum_k x[m, k] * w[n, k] )   x [M, K] (row stride ldx), w [N, K] dense,
  * y [M, N] (row stride ldy).  nn.Linear without bias: wqkv / wo (utils.py:191, 258), w1 / w2
  * (utils.py:146, 148), wqkv1 (utils.py:311), output (gpt_ladder_TP.py:283).
@@ -91,8 +101,9 @@ int lr_linear(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, i
 
 /* lr_linear with the launch configuration of the GEMV given by the caller instead of chosen from
  * the shape: gemv_cfg = rows per wave * 100 + K-split * 10 + unroll, one of 144, 212, 222, 242, 244,
- * 412, 422, 442 (anything else: 242; 0: the shape heuristic, i.e. lr_linear).  Only consulted where
- * lr_linear would run the GEMV.  No counterpart in the reference: for callers that tune per shape.
+ * 412, 422, 442 (anything else: 242; 0: the shape heuristic, i.e. lr_linear).  A non-zero gemv_cfg also selects
+ * the GEMV for M of 5 to 8, where lr_linear would take the skinny matrix-core GEMM; beyond M = 8 it
+ * is ignored.  No counterpart in the reference: for callers that tune per shape.
  * Results do not depend on it beyond the fp32 summation order. */
 int lr_linear_tuned(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
                     int act_swiglu, int gemv_cfg, lr_stream_t stream);

@@ -15,7 +15,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "gpt_fast", "libladder_hip.so")
-HEADERS = [os.path.join(CSRC, "lr_common.h"), os.path.join(HERE, "..", "include", "ladder_hip.h")]
+HEADERS = [os.path.join(CSRC, h) for h in ("lr_common.h", "skinny_tile.h", "attn_decode_item.h")] + \
+    [os.path.join(HERE, "..", "include", "ladder_hip.h")]
 
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",

@@ -146,6 +146,107 @@ extern "C" int lr_add_rmsnorm(const void* resid_in, const void* d1, const void* 
   return lr_launch_status();
 }
 
+// ------------------------------------------------------------------------------------ both norms of a ladder block
+// r1 = bf16(r + d1), n1 = norm(r1) * g1;  r2 = bf16(r1 + d2), n2 = norm(r2) * g2;  r <- r2.
+// In the ladder schedule the MLP's input does not contain the attention output of the same block, so
+// both residual updates and both norms of a block can be done before either module runs.
+__global__ __launch_bounds__(256) void k_ladder_norms(const u16* __restrict__ rin, const u16* __restrict__ d1,
+                                                      const u16* __restrict__ d2, const u16* __restrict__ g1,
+                                                      const u16* __restrict__ g2, u16* rout, u16* __restrict__ n1,
+                                                      u16* __restrict__ n2, int dim, float eps) {
+  __shared__ float red[8];
+  const int tid = threadIdx.x;
+  const int64_t base = (int64_t)blockIdx.x * dim;
+  uint4 qr[NORM_MAXIT], q1[NORM_MAXIT], q2[NORM_MAXIT], qg1[NORM_MAXIT], qg2[NORM_MAXIT];
+#pragma unroll
+  for (int it = 0; it < NORM_MAXIT; ++it) {
+    const int c0 = (tid + it * 256) * 8;
+    if (it * 256 * 8 >= dim) break;  // uniform
+    const int c = c0 < dim ? c0 : 0;
+    qr[it] = ld16(rin + base + c);
+    q1[it] = d1 ? ld16(d1 + base + c) : make_uint4(0, 0, 0, 0);
+    q2[it] = d2 ? ld16(d2 + base + c) : make_uint4(0, 0, 0, 0);
+    qg1[it] = ld16(g1 + c);
+    qg2[it] = ld16(g2 + c);
+  }
+  float ss1 = 0.0f, ss2 = 0.0f;
+#pragma unroll
+  for (int it = 0; it < NORM_MAXIT; ++it) {
+    const int c = (tid + it * 256) * 8;
+    if (it * 256 * 8 >= dim) break;
+    float r[8], t[8];
+    unpack8(qr[it], r);
+    if (d1) {
+      unpack8(q1[it], t);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) r[j] = round_bf(r[j] + t[j]);
+    }
+    qr[it] = pack8(r);  // r1, exact in bf16
+    if (c < dim) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss1 += r[j] * r[j];
+    }
+    if (d2) {
+      unpack8(q2[it], t);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) r[j] = round_bf(r[j] + t[j]);
+    }
+    q2[it] = pack8(r);  // r2
+    if (c < dim) {
+      st16(rout + base + c, q2[it]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss2 += r[j] * r[j];
+    }
+  }
+  ss1 = wave_sum(ss1);
+  ss2 = wave_sum(ss2);
+  if ((tid & 63) == 0) {
+    red[tid >> 6] = ss1;
+    red[4 + (tid >> 6)] = ss2;
+  }
+  __syncthreads();
+  const float inv1 = rsqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)dim + eps);
+  const float inv2 = rsqrtf(((red[4] + red[5]) + (red[6] + red[7])) / (float)dim + eps);
+#pragma unroll
+  for (int it = 0; it < NORM_MAXIT; ++it) {
+    const int c = (tid + it * 256) * 8;
+    if (it * 256 * 8 >= dim) break;
+    if (c < dim) {
+      float r[8], g[8], o[8];
+      unpack8(qr[it], r);
+      unpack8(qg1[it], g);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = round_bf(r[j] * inv1) * g[j];
+      st16(n1 + base + c, pack8(o));
+      unpack8(q2[it], r);
+      unpack8(qg2[it], g);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = round_bf(r[j] * inv2) * g[j];
+      st16(n2 + base + c, pack8(o));
+    }
+  }
+}
+
+extern "C" int lr_ladder_norms(const void* resid_in, const void* d1, const void* d2, const void* gain1, const void* gain2,
+                               void* resid_out, void* normed1, void* normed2, int rows, int dim, float eps,
+                               lr_stream_t stream) {
+  LR_REQUIRE_PTR(resid_in);
+  LR_REQUIRE_PTR(gain1);
+  LR_REQUIRE_PTR(gain2);
+  LR_REQUIRE_PTR(resid_out);
+  LR_REQUIRE_PTR(normed1);
+  LR_REQUIRE_PTR(normed2);
+  LR_OPTIONAL_PTR(d1);
+  LR_OPTIONAL_PTR(d2);
+  if (rows <= 0 || dim <= 0) return LR_E_SHAPE;
+  if (dim % 8) return LR_E_ALIGN;
+  if (dim > 256 * 8 * NORM_MAXIT) return LR_E_UNSUPPORTED;
+  k_ladder_norms<<<dim3(rows), dim3(256), 0, (hipStream_t)stream>>>(
+      (const u16*)resid_in, (const u16*)d1, (const u16*)d2, (const u16*)gain1, (const u16*)gain2, (u16*)resid_out,
+      (u16*)normed1, (u16*)normed2, dim, eps);
+  return lr_launch_status();
+}
+
 // ------------------------------------------------------------------------------------ SwiGLU
 __global__ __launch_bounds__(256) void k_swiglu(const u16* __restrict__ h, int64_t ldh, u16* __restrict__ out, int I) {
   const int row = blockIdx.y;

@@ -20,6 +20,8 @@ _PROTOS = {
     "lr_add": (c_int, [c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p]),
     "lr_add_rmsnorm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float,
                                c_void_p]),
+    "lr_ladder_norms": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                c_float, c_void_p]),
     "lr_linear": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
     "lr_linear_tuned": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int,
                                 c_void_p]),
@@ -144,6 +146,18 @@ def add_rmsnorm(resid_in, d1, d2, gain, resid_out, normed_out, eps: float):
     _check(load().lr_add_rmsnorm(_dev(resid_in), p(d1), p(d2), _dev(gain), p(resid_out), _dev(normed_out), rows, dim,
                                  float(eps), _stream()), "lr_add_rmsnorm")
     return normed_out
+
+
+def ladder_norms(resid_in, d1, d2, gain1, gain2, resid_out, normed1, normed2, eps: float):
+    """Both residual updates and both norms of a ladder block (lr_ladder_norms)."""
+    dim = resid_in.shape[-1]
+    rows = resid_in.numel() // dim
+    for t in (resid_in, d1, d2, resid_out, normed1, normed2):
+        assert t is None or (t.is_contiguous() and t.numel() == rows * dim)
+    assert gain1.numel() == dim and gain2.numel() == dim
+    p = lambda t: None if t is None else _dev(t)
+    _check(load().lr_ladder_norms(_dev(resid_in), p(d1), p(d2), _dev(gain1), _dev(gain2), _dev(resid_out), _dev(normed1),
+                                  _dev(normed2), rows, dim, float(eps), _stream()), "lr_ladder_norms")
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, act_swiglu: bool = False, gemv_cfg: int = 0):

@@ -28,6 +28,7 @@ class Workspace:
         self.B, self.S, self.rows = B, S, rows
         self.x = e(rows, D)        # residual stream
         self.xn = e(rows, D)       # normed input of the current module
+        self.xn2 = e(rows, D) if S == 1 else None   # decode: the MLP's normed input while attention runs beside it
         self.a = e(rows, D)        # attention partial sum (pending in the ladder schedule)
         self.m = e(rows, D)        # MLP partial sum
         self.qkv = e(rows, fused_width)
@@ -175,9 +176,9 @@ class GPTBase(nn.Module):
             _hip.attn_prefill(ws.qkv, kc, vc, pos, ws.y, B, S, Hq, Hkv, hd)
         _hip.module_linear(ws.y, blk.attention.wo, out)
 
-    def _mlp(self, ws: Workspace, blk, out: Tensor):
+    def _mlp(self, ws: Workspace, blk, out: Tensor, xn: Optional[Tensor] = None):
         ff = blk.feed_forward
-        _hip.module_linear(ws.xn, ff.w1, ws.h)
+        _hip.module_linear(ws.xn if xn is None else xn, ff.w1, ws.h)
         _hip.module_linear_swiglu(ws.h, ff.w2, out, ws.act)
 
     # -- greedy decoding helper ---------------------------------------------------------------------

@@ -114,9 +114,47 @@ class GPTLadder(GPTBase):
             return ws.next_token  # already chosen inside the fused step
         return super().greedy_next(logits)
 
+    # Decode through the per-op kernels: run the attention chain and the MLP chain of a block on two streams.
+    # Off by default: as parallel branches of a captured graph the chains do overlap, but every hand-over between
+    # the two hardware queues costs more than the attention chain's latency that it hides (measured on the 70B rank
+    # shard, ms per step with / without: batch 8 8.6 / 8.3, batch 64 18.2 / 18.8).  Putting one step of each chain
+    # into the same grid instead (wqkv beside w1, attention beside w2) was slower still: 10.3 ms at batch 8.
+    overlap_modules = False
+
+    def _run_layers_decode(self, ws: Workspace, pos: Tensor):
+        """Decode step (S == 1) of an all-ladder model through the per-op kernels: one launch does both residual
+        updates and both norms of a block (lr_ladder_norms: the MLP's input does not contain the block's own
+        attention output), then the attention chain (wqkv, RoPE + cache write, attention, wo) and the MLP chain
+        (w1, SwiGLU, w2) -- one after the other, or on two streams where the reference overlaps an all-reduce with
+        the next module (gpt_ladder_TP.py:339-349)."""
+        eps = self.config.norm_eps
+        main = side = None
+        if self.overlap_modules:
+            main = torch.cuda.current_stream()
+            side = getattr(self, "_side_stream", None)
+            if side is None or side.device != main.device:
+                side = self._side_stream = torch.cuda.Stream(device=main.device)
+        pending_a = pending_m = None
+        for blk in self.layers:
+            _hip.ladder_norms(ws.x, pending_a, pending_m, blk.attention_norm.weight, blk.ffn_norm.weight, ws.x, ws.xn,
+                              ws.xn2, eps)
+            if side is not None:
+                side.wait_stream(main)
+                with torch.cuda.stream(side):
+                    self._mlp(ws, blk, ws.m, ws.xn2)
+                self._attention(ws, blk, pos, blk.attention.wqkv, ws.a)
+                main.wait_stream(side)
+            else:
+                self._attention(ws, blk, pos, blk.attention.wqkv, ws.a)
+                self._mlp(ws, blk, ws.m, ws.xn2)
+            pending_a, pending_m = ws.a, ws.m
+        return pending_a, pending_m
+
     def _run_layers(self, ws: Workspace, pos: Tensor):
         cfg = self.config
         eps = cfg.norm_eps
+        if ws.S == 1 and cfg.ladder_layers is None:
+            return self._run_layers_decode(ws, pos)
         pending_a = pending_m = None  # the reference starts from zero tensors; adding zero is the identity
         for i, blk in enumerate(self.layers):
             if cfg.is_ladder_layer(i):

@@ -179,6 +179,18 @@ def test_tiny_ladder_fused_and_per_op_decode(B, fused):
     assert stats["fused_step_used"] == fused
 
 
+@pytest.mark.parametrize("B", [1, 3, 6])
+@pytest.mark.parametrize("mode", ["plain", "two_streams"])
+def test_tiny_ladder_per_op_decode_modes(B, mode):
+    """The per-op decode path of the ladder model: one stream (the default), or the attention and the MLP chain
+    of a block on two streams."""
+    model = build("ladder", **dict(TINY, dim=512, n_head=8, n_local_heads=2, intermediate_size=640))
+    model.overlap_modules = mode == "two_streams"
+    stats = run_parity(model, "ladder", B=B, T=20, new=12, fused=False)
+    print(B, mode, stats)
+    check(stats)
+
+
 def test_tiny_ladder_fused_head_dim_128_many_kv_heads():
     kw = dict(TINY, block_size=128, n_head=8, n_local_heads=2, dim=1024, intermediate_size=768, n_layer=2,
               vocab_size=1000)

@@ -246,6 +246,28 @@ def test_rope_kv_write_exact(hip, hd, Hq, Hkv, gathered):
     assert torch.equal(work[..., Hq * hd:], torch.cat([k, v], -1))   # k and v columns are left as they were
 
 
+@pytest.mark.parametrize("rows,dim", [(1, 8192), (8, 8192), (64, 4096), (3, 2048), (16, 16384), (5, 264)])
+@pytest.mark.parametrize("first_block", [False, True])
+def test_ladder_norms_equals_two_add_rmsnorm_calls(hip, rows, dim, first_block):
+    """lr_ladder_norms (both residual updates + both norms of a block in one launch) must give, bit for bit, what
+    two lr_add_rmsnorm calls give, and match the oracle's block prologue (gpt_ladder_TP.py:326-354)."""
+    x, d1, d2 = rnd(rows, dim, seed=50), rnd(rows, dim, seed=51, scale=0.3), rnd(rows, dim, seed=52, scale=0.3)
+    g1, g2 = rnd(dim, seed=53), rnd(dim, seed=54)
+    if first_block:
+        d1 = d2 = None
+    r_ref, n1_ref, n2_ref = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+    hip.add_rmsnorm(x, d1, None, g1, r_ref, n1_ref, 1e-5)
+    hip.add_rmsnorm(r_ref, d2, None, g2, r_ref, n2_ref, 1e-5)
+    r, n1, n2 = x.clone(), torch.empty_like(x), torch.empty_like(x)
+    hip.ladder_norms(r, d1, d2, g1, g2, r, n1, n2, 1e-5)       # residual updated in place
+    assert torch.equal(r, r_ref) and torch.equal(n1, n1_ref) and torch.equal(n2, n2_ref)
+    r1 = x if first_block else x + d1
+    r2 = r1 if first_block else r1 + d2
+    assert torch.equal(r, r2)
+    assert_close_ulp(n1, O.rms_norm(r1, g1, 1e-5), max_ulp=2, max_frac=0.05, what="ladder_norms n1")
+    assert_close_ulp(n2, O.rms_norm(r2, g2, 1e-5), max_ulp=2, max_frac=0.05, what="ladder_norms n2")
+
+
 # ------------------------------------------------------------------------------------ weight-only fp8 linear
 
 def test_linear_fp8_decodes_every_e4m3_value_exactly(hip):
