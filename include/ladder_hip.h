@@ -89,11 +89,11 @@ int lr_ladder_norms(const void* resid_in, const void* d1, const void* d2, const 
  * y [M, N] (row stride ldy).  nn.Linear without bias: wqkv / wo (utils.py:191, 258), w1 / w2
  * (utils.py:146, 148), wqkv1 (utils.py:311), output (gpt_ladder_TP.py:283).
  * K % 8 == 0.  The kernel is chosen from the shape: M <= 4 (and M <= 8 with act_swiglu) the
- * weight-streaming GEMV (v_dot2 on packed pairs, every weight read once); 4 < M <= 8 on a matrix
- * with few rows two GEMV passes of four rows; 4 < M <= 64 the skinny matrix-core GEMM (32 weight
- * rows per workgroup, K split over the waves); M >= 512 on a large enough grid the 256 x 256 tile
- * matrix-core GEMM; everything else the 128 x 128 tile matrix-core GEMM.  All of them accumulate
- * in fp32 and round once; the summation order, hence the last bit, depends on the kernel.
+ * weight-streaming GEMV (v_dot2 on packed pairs, every weight read once); 4 < M <= 64 the
+ * weight-streaming matrix-core kernel of lr_linear_multi; M >= 512 on a large enough grid the
+ * 256 x 256 tile matrix-core GEMM; everything else the 128 x 128 tile matrix-core GEMM.  All of
+ * them accumulate in fp32 and round once; the summation order, hence the last bit, depends on the
+ * kernel.
  * act_swiglu != 0: x is taken to be [M, 2K] = [u | g] (row stride ldx) and the kernel consumes
  * bf16( bf16(silu(g)) * u ) in its place -- w2(silu(g) * u), utils.py:147-148. */
 int lr_linear(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K, int act_swiglu,
@@ -101,12 +101,32 @@ int lr_linear(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, i
 
 /* lr_linear with the launch configuration of the GEMV given by the caller instead of chosen from
  * the shape: gemv_cfg = rows per wave * 100 + K-split * 10 + unroll, one of 144, 212, 222, 242, 244,
- * 412, 422, 442 (anything else: 242; 0: the shape heuristic, i.e. lr_linear).  A non-zero gemv_cfg also selects
- * the GEMV for M of 5 to 8, where lr_linear would take the skinny matrix-core GEMM; beyond M = 8 it
- * is ignored.  No counterpart in the reference: for callers that tune per shape.
+ * 412, 422, 442 (anything else: 242; 0: the shape heuristic, i.e. lr_linear).  A non-zero gemv_cfg
+ * also selects the GEMV for M of 5 to 8, where lr_linear would take the matrix-core streaming
+ * kernel; beyond M = 8 it is ignored.  No counterpart in the reference: for callers that tune per shape.
  * Results do not depend on it beyond the fp32 summation order. */
 int lr_linear_tuned(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
                     int act_swiglu, int gemv_cfg, lr_stream_t stream);
+
+/* Up to two projections of the same M input rows (M <= 64) in ONE launch of the weight-streaming
+ * kernel, e.g. the fused q/k/v projection (utils.py:188) next to the MLP's up/gate projection
+ * (utils.py:142-148) in a ladder block, whose inputs are both ready before either runs
+ * (gpt_ladder_TP.py:323-349).  Per projection: y[M, N] = x[M, K] w[N, K]^T as in lr_linear
+ * (epilogue LR_EPI_NONE), or, for a weight holding [up; gate] rows (N = 2 I, the layout of
+ * feed_forward.w1), y[M, I] = bf16( bf16(silu(g)) * u ) with u, g the bf16-rounded projections
+ * (LR_EPI_SWIGLU: utils.py:145-148 without the [M, 2 I] round trip).  Sums are fp32, added in a
+ * fixed order.  The reference has no such call; it is what its compiled decode graph amounts to. */
+enum { LR_EPI_NONE = 0, LR_EPI_SWIGLU = 1 };
+typedef struct lr_projection {
+  const void* x; /* [M, K] bf16, row stride ldx */
+  int64_t ldx;
+  const void* w; /* [N, K] bf16, dense */
+  void* y;       /* [M, N] (or [M, N / 2]) bf16, row stride ldy */
+  int64_t ldy;
+  int32_t N, K;
+  int32_t epilogue;
+} lr_projection_t;
+int lr_linear_multi(const lr_projection_t* projections, int n_projections, int M, lr_stream_t stream);
 
 /* Weight-only fp8 linear:  y[m, n] = bf16( bf16( sum_k x[m, k] * w8[n, k] ) * scales[n] ).
  * w8 [N, K] dense float8 e4m3 (OCP "e4m3fn": bias 7, no infinities, max 448), one byte per weight;

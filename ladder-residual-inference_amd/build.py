@@ -15,7 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "gpt_fast", "libladder_hip.so")
-HEADERS = [os.path.join(CSRC, h) for h in ("lr_common.h", "skinny_tile.h", "attn_decode_item.h")] + \
+HEADERS = [os.path.join(CSRC, h) for h in ("lr_common.h", "attn_decode_item.h")] + \
     [os.path.join(HERE, "..", "include", "ladder_hip.h")]
 
 FLAGS = [

@@ -8,7 +8,6 @@
 // reads that deliver exactly the 8 consecutive k an MFMA lane feeds.  LDS is double-buffered and
 // the global loads of tile t+1 are in flight while tile t is multiplied.
 #include "lr_common.h"
-#include "skinny_tile.h"
 #include <type_traits>
 
 int lr_gemv_dispatch(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
@@ -308,14 +307,6 @@ static int launch_gemm_big(const void* x, int64_t ldx, const void* w, void* y, i
   return lr_launch_status();
 }
 
-template <int MT>
-__global__ __launch_bounds__(SW * 64) void k_gemm_skinny(const u16* __restrict__ x, int64_t ldx,
-                                                         const u16* __restrict__ w, u16* __restrict__ y, int64_t ldy,
-                                                         int M, int N, int K) {
-  __shared__ __attribute__((aligned(16))) float red[SW * (MT / 32) * 16 * 64];
-  skinny_tile<MT>(x, ldx, w, y, ldy, M, N, K, blockIdx.x * SN, red);
-}
-
 extern "C" int lr_linear_tuned(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
                                int act_swiglu, int gemv_cfg, lr_stream_t stream) {
   LR_REQUIRE_PTR(x);
@@ -327,21 +318,12 @@ extern "C" int lr_linear_tuned(const void* x, int64_t ldx, const void* w, void* 
   hipStream_t s = (hipStream_t)stream;
   if (M <= 4 || ((act_swiglu || gemv_cfg) && M <= 8))
     return lr_gemv_dispatch(x, ldx, w, y, ldy, M, N, K, act_swiglu, gemv_cfg, s);
-  if (!act_swiglu && M <= 8 && (N + SN - 1) / SN < 96) {
-    // few weight rows (the wqkv of a rank shard): 32-row workgroups would leave most CUs idle, so the
-    // GEMV kernel (a row per wave, every CU busy) runs twice, four input rows each; the second pass
-    // finds the weights in the memory-side cache
-    const int rc = lr_gemv_dispatch(x, ldx, w, y, ldy, 4, N, K, 0, 0, s);
-    if (rc != LR_OK) return rc;
-    return lr_gemv_dispatch((const u16*)x + 4 * ldx, ldx, w, (u16*)y + 4 * ldy, ldy, M - 4, N, K, 0, 0, s);
-  }
-  if (!act_swiglu && M <= 64 && ldy % 2 == 0 && (int64_t)64 * ldx * 2 < 0x7fffffff && (int64_t)SN * K * 2 < 0x7fffffff) {
-    const dim3 sgrid((N + SN - 1) / SN);
-    if (M <= 32)
-      k_gemm_skinny<32><<<sgrid, dim3(SW * 64), 0, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy, M, N, K);
-    else
-      k_gemm_skinny<64><<<sgrid, dim3(SW * 64), 0, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy, M, N, K);
-    return lr_launch_status();
+  if (!act_swiglu && M <= 64) {
+    // decode batches: the weight-streaming matrix-core kernel (stream_gemm.hip); shapes it declines fall through
+    lr_projection_t pr;
+    pr.x = x; pr.ldx = ldx; pr.w = w; pr.y = y; pr.ldy = ldy; pr.N = N; pr.K = K; pr.epilogue = LR_EPI_NONE;
+    const int rc = lr_linear_multi(&pr, 1, M, stream);
+    if (rc != LR_E_UNSUPPORTED) return rc;
   }
   if (!act_swiglu && M >= 512 && N >= 256 && ((M + GM - 1) / GM) * ((N + GN - 1) / GN) >= 192 &&
       (int64_t)GM * ldx * 2 < 0x7fffffff && (int64_t)GN * K * 2 < 0x7fffffff)

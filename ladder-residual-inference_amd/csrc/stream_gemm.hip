@@ -1,0 +1,260 @@
+// Weight-streaming GEMM for decode batches (up to 64 input rows):  y[m, n] = bf16( sum_k x[m, k] * w[n, k] ).
+//
+// The weights are read once, in whole cache lines: a load instruction covers 4 weight rows x 256
+// contiguous bytes (16 lanes x 16 bytes per row), never a fraction of a line that another
+// instruction would have to find in a cache again.  That is the layout a matrix-vector kernel
+// streams in, not the one the matrix cores want (there a lane feeds 8 consecutive k of ITS OWN row,
+// 16 different rows per instruction), so every chunk takes one trip through a wave-private piece of
+// LDS: written row-major as it arrives, read back as v_mfma_f32_16x16x32_bf16 A fragments.  Rows
+// are padded by 16 bytes, which puts the 16 rows of a fragment read on 16 different bank groups.
+// No workgroup barrier is involved: the LDS unit executes a wave's instructions in order.
+//
+// A workgroup (4 waves, one per SIMD, so each has the whole register budget) owns a band of up to
+// 32 weight rows -- the number of rows is chosen so that every CU gets the same share -- and its
+// waves split K in 128-element chunks (wave w takes chunks w, w + 4, ...: together they read 1 KiB
+// contiguous per row and round).  Each wave keeps 4 chunks of weights (32 KiB) in flight in
+// registers, 128 KiB per CU.  The input rows come from L2 straight into B-fragment layout, one
+// chunk ahead.  The waves' partial sums meet in LDS and are added in a fixed order.
+//
+// Two projections that read the same layer input can share one launch (the band index selects the
+// projection), and a projection whose weight holds [up; gate] rows can take the band as row PAIRS
+// and store bf16(bf16(silu(g)) * u) instead of u and g.
+#include "lr_common.h"
+
+namespace {
+
+constexpr int KC = 128;        // k elements per chunk
+constexpr int NWV = 4;         // waves per workgroup
+constexpr int SETS = 4;        // weight chunks in flight per wave
+constexpr int LROW = KC + 8;   // LDS row length in elements (272 bytes)
+constexpr int OOB = (int)0x80000000;  // a buffer offset beyond every resource: the load returns zero, untouched memory
+#ifndef LR_SG_W_AUX
+#define LR_SG_W_AUX 2          // weights: non-temporal (every line is used exactly once)
+#endif
+
+struct Proj {
+  const u16* x;
+  const u16* w;
+  u16* y;
+  int64_t ldx, ldy;
+  int N, K;      // weight rows, row length
+  int rpw;       // rows (row pairs if pair_off) per workgroup
+  int pair_off;  // 0, or the distance from an up row to its gate row (= outputs)
+  int nwg;       // workgroups of this projection
+};
+
+template <int MT, int UNITS>
+__global__ __launch_bounds__(NWV * 64) void k_stream_gemm(const Proj p0, const Proj p1, const int M) {
+  constexpr int MTILES = MT / 16, KS = KC / 32, NLD = UNITS * 4;
+  constexpr int NV = UNITS * MTILES * 4;  // accumulator registers per lane
+  __shared__ __attribute__((aligned(16))) u16 lds[NWV][UNITS * 16 * LROW];
+  static_assert(sizeof(float) * NV * 64 <= sizeof(u16) * UNITS * 16 * LROW, "the partial sums reuse the wave's LDS piece");
+
+  const bool second = (int)blockIdx.x >= p0.nwg;
+  const u16* const xg = second ? p1.x : p0.x;
+  const u16* const wg_ = second ? p1.w : p0.w;
+  u16* const yg = second ? p1.y : p0.y;
+  const int64_t ldx = second ? p1.ldx : p0.ldx, ldy = second ? p1.ldy : p0.ldy;
+  const int N = second ? p1.N : p0.N, K = second ? p1.K : p0.K, rpw = second ? p1.rpw : p0.rpw;
+  const int pair_off = second ? p1.pair_off : p0.pair_off;
+  const int band = second ? (int)blockIdx.x - p0.nwg : (int)blockIdx.x;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l16 = lane & 15, l4 = lane >> 4;
+  const int n_out = pair_off ? pair_off : N;         // output columns
+  const int n0 = band * rpw;                          // first row (pair) of the band
+  const int nrows = n_out - n0 < rpw ? n_out - n0 : rpw;
+
+  // ---- lane constants of the weight loads: instruction i covers band rows 4 i .. 4 i + 3 (in pair mode
+  //      unit 0 holds the up rows, unit 1 the gate rows of the same pairs)
+  const __amdgpu_buffer_rsrc_t wres =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<u16*>(wg_ + (int64_t)n0 * K), 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc(const_cast<u16*>(xg), 0, 0x7fffffff, 0x00020000);
+  int woff[NLD];
+#pragma unroll
+  for (int i = 0; i < NLD; ++i) {
+    const int r = 4 * i + l4;  // row inside the LDS piece
+    int rr = r, extra = 0;
+    if (pair_off && r >= 16) { rr = r - 16; extra = pair_off; }
+    woff[i] = rr < nrows ? (int)(((int64_t)(extra + rr) * K + l16 * 8) * 2) : OOB;
+  }
+  int xoff[MTILES];
+#pragma unroll
+  for (int mt = 0; mt < MTILES; ++mt) {
+    const int m = mt * 16 + l16;
+    xoff[mt] = m < M ? (int)((m * ldx + l4 * 8) * 2) : OOB;
+  }
+  u16* const my = lds[wave];
+
+  u32x4_t wr[SETS][NLD];
+  u32x4_t xr[2][MTILES][KS];
+  f32x4_t acc[UNITS][MTILES];
+#pragma unroll
+  for (int u = 0; u < UNITS; ++u)
+#pragma unroll
+    for (int mt = 0; mt < MTILES; ++mt) acc[u][mt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+  // chunk ci of this wave starts at k0 = (ci * NWV + wave) * KC; what lies beyond K reads as zero (no
+  // branch around a load: the number of loads in flight is fixed, so the waits between chunks are exact)
+  auto issue_w = [&](int ci, u32x4_t (&dst)[NLD]) {
+    const int k0 = (ci * NWV + wave) * KC;
+    const bool kok = k0 + l16 * 8 < K;
+#pragma unroll
+    for (int i = 0; i < NLD; ++i)
+      dst[i] = __builtin_amdgcn_raw_buffer_load_b128(wres, (kok && woff[i] != OOB) ? woff[i] : OOB, k0 * 2, LR_SG_W_AUX);
+  };
+  auto issue_x = [&](int ci, u32x4_t (&dst)[MTILES][KS]) {
+    const int k0 = (ci * NWV + wave) * KC;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const bool kok = k0 + ks * 32 + l4 * 8 < K;
+#pragma unroll
+      for (int mt = 0; mt < MTILES; ++mt)
+        dst[mt][ks] = __builtin_amdgcn_raw_buffer_load_b128(xres, (kok && xoff[mt] != OOB) ? xoff[mt] : OOB,
+                                                           (k0 + ks * 32) * 2, 0);
+    }
+  };
+
+  const int nck = (K + KC - 1) / KC;
+  const int nch = wave < nck ? (nck - wave + NWV - 1) / NWV : 0;  // chunks of this wave
+  issue_x(0, xr[0]);
+#pragma unroll
+  for (int s = 0; s < SETS; ++s) issue_w(s, wr[s]);
+  for (int c0 = 0; c0 < nch; c0 += SETS) {
+#pragma unroll
+    for (int s = 0; s < SETS; ++s) {
+      const int ci = c0 + s;
+      issue_x(ci + 1, xr[(s + 1) & 1]);
+      // ---- this chunk's weights: registers -> LDS (row-major) -> A fragments
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int i = 0; i < NLD; ++i)
+        *reinterpret_cast<u32x4_t*>(my + (4 * i + l4) * LROW + l16 * 8) = wr[s][i];
+      asm volatile("" ::: "memory");
+      bf16x8_t af[UNITS][KS];
+#pragma unroll
+      for (int u = 0; u < UNITS; ++u)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          af[u][ks] = *reinterpret_cast<const bf16x8_t*>(my + (16 * u + l16) * LROW + ks * 32 + l4 * 8);
+      asm volatile("" ::: "memory");
+      issue_w(ci + SETS, wr[s]);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int mt = 0; mt < MTILES; ++mt) {
+          const bf16x8_t bx = __builtin_bit_cast(bf16x8_t, xr[s & 1][mt][ks]);
+#pragma unroll
+          for (int u = 0; u < UNITS; ++u)
+            acc[u][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[u][ks], bx, acc[u][mt], 0, 0, 0);
+        }
+    }
+  }
+
+  // ---- the waves' partial sums meet in LDS (accumulator element e of tile (u, mt): band row
+  //      16 u + 4 (lane / 16) + e, input row 16 mt + lane % 16) and are added in wave order
+  __syncthreads();
+  float* const red = reinterpret_cast<float*>(&lds[0][0]);
+  constexpr int WSTRIDE = UNITS * 16 * LROW / 2;  // floats per wave piece
+#pragma unroll
+  for (int u = 0; u < UNITS; ++u)
+#pragma unroll
+    for (int mt = 0; mt < MTILES; ++mt)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) red[wave * WSTRIDE + ((u * MTILES + mt) * 4 + e) * 64 + lane] = acc[u][mt][e];
+  __syncthreads();
+  const int rows_out = pair_off ? 16 : 16 * UNITS;
+  for (int o = tid; o < rows_out * MT; o += NWV * 64) {
+    const int r = o % rows_out, m = o / rows_out;
+    if (r >= nrows || m >= M) continue;
+    const int mt = m >> 4, ln = ((r & 15) >> 2) * 16 + (m & 15), e = r & 3, u = r >> 4;
+    float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+    for (int wv = 0; wv < NWV; ++wv) s0 += red[wv * WSTRIDE + ((u * MTILES + mt) * 4 + e) * 64 + ln];
+    if (pair_off) {
+      if (UNITS == 2) {
+#pragma unroll
+        for (int wv = 0; wv < NWV; ++wv) s1 += red[wv * WSTRIDE + ((MTILES + mt) * 4 + e) * 64 + ln];
+      }
+      yg[(int64_t)m * ldy + n0 + r] = f_to_bf(swiglu_bf(round_bf(s0), round_bf(s1)));
+    } else {
+      yg[(int64_t)m * ldy + n0 + r] = f_to_bf(s0);
+    }
+  }
+}
+
+static int num_cus() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0;
+    n = prop.multiProcessorCount;
+  }
+  return n;
+}
+
+// Rows per workgroup: the rows are spread evenly over whole rounds of the CUs, at most `cap` per
+// workgroup; with few weight rows and many input rows a band is not made thinner than `floor_rows`
+// (every band re-reads all input rows from L2).
+static void plan(Proj& p, int M, int cap, int ncu) {
+  const int items = p.pair_off ? p.pair_off : p.N;
+  const int rounds = (items + ncu * cap - 1) / (ncu * cap);
+  int rpw = (items + ncu * rounds - 1) / (ncu * rounds);
+  const int floor_rows = M > 32 ? 16 : (M > 16 ? 8 : 4);
+  if (rpw < floor_rows) rpw = floor_rows;
+  if (rpw > cap) rpw = cap;
+  p.rpw = rpw;
+  p.nwg = (items + rpw - 1) / rpw;
+}
+
+template <int MT>
+static void launch(Proj& a, Proj& b, int M, int units, hipStream_t s) {
+  const dim3 grid((unsigned)(a.nwg + b.nwg));
+  if (units == 2) k_stream_gemm<MT, 2><<<grid, dim3(NWV * 64), 0, s>>>(a, b, M);
+  else k_stream_gemm<MT, 1><<<grid, dim3(NWV * 64), 0, s>>>(a, b, M);
+}
+
+}  // namespace
+
+extern "C" int lr_linear_multi(const lr_projection_t* proj, int n_proj, int M, lr_stream_t stream) {
+  if (proj == nullptr) return LR_E_NULL;
+  if (n_proj < 1 || n_proj > 2 || M < 1) return LR_E_SHAPE;
+  if (M > 64) return LR_E_UNSUPPORTED;
+  Proj pr[2] = {};
+  bool any_pair = false;
+  for (int i = 0; i < n_proj; ++i) {
+    const lr_projection_t& q = proj[i];
+    LR_REQUIRE_PTR(q.x);
+    LR_REQUIRE_PTR(q.w);
+    LR_REQUIRE_PTR(q.y);
+    if (q.N <= 0 || q.K <= 0 || q.ldx < q.K) return LR_E_SHAPE;
+    if (q.epilogue != LR_EPI_NONE && q.epilogue != LR_EPI_SWIGLU) return LR_E_SHAPE;
+    const bool pair = q.epilogue == LR_EPI_SWIGLU;
+    if (pair && q.N % 2) return LR_E_SHAPE;
+    if (q.ldy < (pair ? q.N / 2 : q.N)) return LR_E_SHAPE;
+    if (q.K % 8 || q.ldx % 8) return LR_E_ALIGN;
+    // offsets inside a band and inside the input rows are 32-bit
+    if ((int64_t)64 * q.ldx * 2 >= 0x7fffffff || ((int64_t)(pair ? q.N / 2 : 0) + 64) * q.K * 2 >= 0x7fffffff)
+      return LR_E_UNSUPPORTED;
+    Proj& p = pr[i];
+    p.x = (const u16*)q.x; p.w = (const u16*)q.w; p.y = (u16*)q.y;
+    p.ldx = q.ldx; p.ldy = q.ldy; p.N = q.N; p.K = q.K;
+    p.pair_off = pair ? q.N / 2 : 0;
+    any_pair = any_pair || pair;
+  }
+  const int ncu = num_cus();
+  if (ncu < 1) return LR_E_LAUNCH;
+  bool all_thin = true;
+  for (int i = 0; i < n_proj; ++i)
+    if (pr[i].N > 16 * ncu) all_thin = false;
+  // one 16-row unit per workgroup when every CU still gets a band that way; row pairs always take two units
+  const int units = (any_pair || !all_thin) ? 2 : 1;
+  for (int i = 0; i < n_proj; ++i) plan(pr[i], M, pr[i].pair_off ? 16 : 16 * units, ncu);
+  hipStream_t s = (hipStream_t)stream;
+  if (M <= 16) launch<16>(pr[0], pr[1], M, units, s);
+  else if (M <= 32) launch<32>(pr[0], pr[1], M, units, s);
+  else launch<64>(pr[0], pr[1], M, units, s);
+  return lr_launch_status();
+}

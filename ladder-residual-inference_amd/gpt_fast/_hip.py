@@ -25,6 +25,7 @@ _PROTOS = {
     "lr_linear": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
     "lr_linear_tuned": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int,
                                 c_void_p]),
+    "lr_linear_multi": (c_int, [c_void_p, c_int, c_int, c_void_p]),
     "lr_linear_fp8_scratch_bytes": (c_size_t, [c_int, c_int, c_int]),
     "lr_linear_fp8": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p,
                               c_size_t, c_void_p]),
@@ -178,6 +179,32 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, act_swiglu: bool
 
 
 _FP8_SCRATCH = {}
+
+
+class _Projection(ctypes.Structure):   # lr_projection_t
+    _fields_ = [("x", c_void_p), ("ldx", c_int64), ("w", c_void_p), ("y", c_void_p), ("ldy", c_int64),
+                ("N", ctypes.c_int32), ("K", ctypes.c_int32), ("epilogue", ctypes.c_int32)]
+
+
+EPI_NONE, EPI_SWIGLU = 0, 1
+
+
+def linear_multi(*projections):
+    """One launch of the weight-streaming kernel for one or two projections of the same M <= 64 rows.
+    Each projection is (x [M, K], w [N, K], out, epilogue): EPI_NONE -> out [M, N] = x @ w^T;
+    EPI_SWIGLU -> w holds [up; gate] rows and out [M, N / 2] = silu(gate) * up (lr_linear_multi)."""
+    arr = (_Projection * len(projections))()
+    M = None
+    for i, (x, w, out, epi) in enumerate(projections):
+        m, K, ldx = _rows_ld(x)
+        N, Kw = w.shape
+        Mo, No, ldy = _rows_ld(out)
+        assert w.is_contiguous() and Kw == K and Mo == m and No == (N // 2 if epi == EPI_SWIGLU else N), \
+            (x.shape, w.shape, out.shape, epi)
+        assert M is None or M == m
+        M = m
+        arr[i] = _Projection(_dev(x), ldx, _dev(w), _dev(out), ldy, N, K, epi)
+    _check(load().lr_linear_multi(ctypes.cast(arr, c_void_p), len(projections), M, _stream()), "lr_linear_multi")
 
 
 def linear_fp8(x: torch.Tensor, w8: torch.Tensor, scales: torch.Tensor, out: torch.Tensor):

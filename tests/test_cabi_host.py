@@ -61,6 +61,20 @@ def test_validation_precedes_any_device_work(lib):
     assert lib.lr_linear(None, 0, None, None, 0, 1, 8, 8, 0, None) == E_NULL
     assert lib.lr_linear(64, 8, 128, 256, 8, 0, 8, 8, 0, None) == E_SHAPE
     assert lib.lr_argmax(None, 0, None, 1, 8, None) == E_NULL
+    from gpt_fast._hip import _Projection, EPI_SWIGLU
+    import ctypes
+    one = (_Projection * 1)(_Projection(64, 8, 128, 256, 8, 8, 8, 0))
+    ptr = ctypes.cast(one, ctypes.c_void_p)
+    assert lib.lr_linear_multi(None, 1, 1, None) == E_NULL
+    assert lib.lr_linear_multi(ptr, 3, 1, None) == E_SHAPE          # at most two projections
+    assert lib.lr_linear_multi(ptr, 1, 65, None) == -4              # more than 64 rows: unsupported
+    one[0].epilogue = EPI_SWIGLU
+    one[0].N = 7                                                    # [up; gate] rows come in pairs
+    assert lib.lr_linear_multi(ptr, 1, 1, None) == E_SHAPE
+    one[0].N, one[0].K = 8, 12                                      # K % 8
+    assert lib.lr_linear_multi(ptr, 1, 1, None) == E_SHAPE          # ldx < K
+    one[0].ldx = 16
+    assert lib.lr_linear_multi(ptr, 1, 1, None) == E_ALIGN
     assert lib.lr_ladder_decode_step(None, 1, None, None, None, 0, None, 0, None, None, 0, 0, 0, None, 0, None) == E_NULL
     assert lib.lr_ladder_step_workspace_bytes(None, 1) == 0
 

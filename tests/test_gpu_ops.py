@@ -143,21 +143,76 @@ def test_linear_gemv(hip, M, N, K):
     assert_close_ulp(y, F.linear(x, w), max_frac=0.05, what="gemv vs F.linear")
 
 
-@pytest.mark.parametrize("N,K", [(1280, 8192), (7168, 8192), (8192, 3584), (16032, 8192), (4096, 4096), (24, 64),
-                                 (1001, 520), (130, 136)])
-@pytest.mark.parametrize("M", [5, 8, 16, 31, 33, 64])
-def test_linear_skinny_batches(hip, M, N, K):
-    """Decode batches (4 < M <= 64) take the skinny matrix-core GEMM: ragged N, K not a multiple of the
-    128-element tile, M on both sides of the 32-row column tile, a strided output view."""
+@pytest.mark.parametrize("N,K", [(1280, 8192), (8192, 1024), (7168, 8192), (8192, 3584), (16032, 8192), (4096, 4096),
+                                 (4096, 14336), (24, 64), (1001, 520), (130, 136), (33, 8)])
+@pytest.mark.parametrize("M", [5, 8, 16, 17, 31, 33, 64])
+def test_linear_decode_batches(hip, M, N, K):
+    """Decode batches (4 < M <= 64) take the weight-streaming matrix-core kernel: ragged N (bands that end
+    inside a 16-row unit), K not a multiple of the 128-element chunk or shorter than one, M on both sides
+    of the 16-row column tiles, a strided output view."""
     x = rnd(M, K, seed=12)
     w = rnd(N, K, seed=13, scale=0.02)
     y = torch.empty(M, N, dtype=BF, device=DEV)
     hip.linear(x, w, y)
-    assert_close_ulp(y, linear_ref(x, w), what=f"skinny M={M} N={N} K={K}")
+    assert_close_ulp(y, linear_ref(x, w), what=f"decode batch M={M} N={N} K={K}")
     if N % 8 == 0:
         wide = torch.zeros(M, N + 8, dtype=BF, device=DEV)
         hip.linear(x, w, wide[:, :N])
         assert torch.equal(wide[:, :N], y) and bool((wide[:, N:] == 0).all())
+
+
+def swiglu_of_projection_ref(x, w1):
+    """[up; gate] rows -> bf16(bf16(silu(g)) * u) with u, g the projections rounded to bf16 (utils.py:145-148)."""
+    h = linear_ref(x, w1)
+    inter = w1.shape[0] // 2
+    return F.silu(h[:, inter:]) * h[:, :inter]   # feed_forward of the oracle: silu(g) * u on bf16 tensors
+
+
+@pytest.mark.parametrize("M,D,NQ,I", [(8, 8192, 1280, 3584), (64, 8192, 1280, 3584), (16, 4096, 6144, 14336),
+                                      (5, 264, 40, 50), (33, 136, 520, 17), (1, 512, 96, 200), (64, 72, 8, 1000)])
+def test_linear_multi_two_projections_one_launch(hip, M, D, NQ, I):
+    """q/k/v projection next to the up/gate projection with the SwiGLU epilogue, in one launch: each output
+    against the oracle's op on its own input; bands of different heights in the two projections."""
+    xa, xb = rnd(M, D, seed=30), rnd(M, D, seed=31)
+    wq, w1 = rnd(NQ, D, seed=32, scale=0.03), rnd(2 * I, D, seed=33, scale=0.03)
+    q = torch.empty(M, NQ, dtype=BF, device=DEV)
+    act = torch.full((M, I), 3.0, dtype=BF, device=DEV)
+    hip.linear_multi((xa, wq, q, hip.EPI_NONE), (xb, w1, act, hip.EPI_SWIGLU))
+    assert_close_ulp(q, linear_ref(xa, wq), what="multi: plain projection")
+    # u and g may each sit one ulp away from the fp64-rounded projections; the activation amplifies that
+    want = swiglu_of_projection_ref(xb, w1)
+    assert torch.isfinite(act.float()).all()
+    err = (act.float() - want.float()).abs().max().item()
+    assert err <= 2.0 ** -6 * want.float().abs().max().item(), err
+    assert (ulp_diff(act, want) > 1).float().mean().item() < 0.05
+    # the same projections one at a time give the same bits
+    q1, act1 = torch.empty_like(q), torch.empty_like(act)
+    hip.linear_multi((xa, wq, q1, hip.EPI_NONE))
+    hip.linear_multi((xb, w1, act1, hip.EPI_SWIGLU))
+    assert torch.equal(q1, q) and torch.equal(act1, act)
+
+
+def test_linear_multi_swiglu_epilogue_equals_the_two_step_path(hip):
+    """The fused epilogue rounds where the unfused path rounds: w1 -> h (bf16) -> lr_swiglu gives the same bits."""
+    M, D, I = 8, 1024, 520
+    x, w1 = rnd(M, D, seed=34), rnd(2 * I, D, seed=35, scale=0.03)
+    act = torch.empty(M, I, dtype=BF, device=DEV)
+    hip.linear_multi((x, w1, act, hip.EPI_SWIGLU))
+    h = torch.empty(M, 2 * I, dtype=BF, device=DEV)
+    hip.linear_multi((x, w1, h, hip.EPI_NONE))
+    two_step = torch.empty(M, I, dtype=BF, device=DEV)
+    hip.swiglu(h, two_step)
+    assert torch.equal(act, two_step)
+
+
+def test_linear_multi_is_deterministic(hip):
+    x, w = rnd(64, 8192, seed=36), rnd(1280, 8192, seed=37, scale=0.02)
+    ys = []
+    for _ in range(4):
+        y = torch.empty(64, 1280, dtype=BF, device=DEV)
+        hip.linear_multi((x, w, y, hip.EPI_NONE))
+        ys.append(y)
+    assert all(torch.equal(ys[0], t) for t in ys[1:])
 
 
 @pytest.mark.parametrize("cfg", [144, 212, 222, 242, 244, 412, 422, 442])
