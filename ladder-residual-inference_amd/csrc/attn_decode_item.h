@@ -1,9 +1,12 @@
 #pragma once
 #include "lr_common.h"
 
-// ---- how the valid keys are cut into chunks (one workgroup item per chunk, kv head and sequence)
+// ---- how the valid keys are cut into chunks (one workgroup item per chunk, kv head and sequence).
+//      A chunk never exceeds ATT_CHUNK keys: the item then requests all of its K and V rows at once.
+constexpr int ATT_CHUNK = 256;
+
 static inline int attn_nsplit_cap(int Smax) {
-  const int by_len = (Smax + 511) / 512;  // a chunk never exceeds 512 keys (LDS score buffer)
+  const int by_len = (Smax + ATT_CHUNK - 1) / ATT_CHUNK;
   return by_len > 64 ? by_len : 64;
 }
 
@@ -12,19 +15,31 @@ static inline int attn_pick_nsplit(int B, int Hkv, int Smax) {
   int n = (512 + B * Hkv - 1) / (B * Hkv);   // aim at >= 512 workgroups
   const int by_work = (Smax + 63) / 64;      // but at least ~64 keys per chunk at full length
   if (n > by_work) n = by_work;
-  const int by_len = (Smax + 511) / 512;
+  const int by_len = (Smax + ATT_CHUNK - 1) / ATT_CHUNK;
   if (n < by_len) n = by_len;
   if (n < 1) n = 1;
   return n > cap ? cap : n;
 }
 
+// LDS row length of the score buffer: whole 16-key tiles, plus 4 so that the 16 heads a tile's scores are
+// written for do not share a bank
+__host__ __device__ constexpr int attn_sc_ld(int chunk_max) { return ((chunk_max + 15) & ~15) + 4; }
 
 // One (split, kv head, sequence) item of the split-KV decode attention, by 256 lanes (4 waves): scores,
-// softmax statistics and the un-normalised P.V of keys [k0, k1) for all G q heads of the kv head.
-// `smem`: attn_item_lds_floats<HD, G>(chunk_max) floats of LDS.  A device function so that the plain
-// kernel stays a thin wrapper.
+// softmax statistics and the un-normalised P.V of keys [k0, k1) (at most ATT_CHUNK) for all G q heads of
+// the kv head.  `smem`: attn_item_lds_floats<HD, G>(chunk_max) floats of LDS.
+//
+// Every K and V row of the chunk is requested before anything else -- whole rows, 1 KiB contiguous per
+// wave instruction, up to 32 KiB per wave in flight -- so the item costs one memory round trip.  Scores
+// run on the matrix cores: a 16-key tile of K takes a trip through a wave-private piece of LDS (written
+// row-major as loaded, read back as v_mfma_f32_16x16x32_bf16 A fragments, rows padded by 16 bytes), the
+// q heads are the B operand (loaded straight into fragment layout, heads beyond G are zero columns).
+// Softmax statistics and P.V stay in fp32 on the vector units: a lane owns 8 output elements of one key
+// group, so the inner loop has no cross-lane traffic.
 template <int HD, int G>
-__host__ __device__ constexpr int attn_item_lds_floats(int chunk_max) { return G * HD * 5 + G * chunk_max + 2 * G; }
+__host__ __device__ constexpr int attn_item_lds_floats(int chunk_max) {
+  return (4 * G * HD > 32 * (HD + 8) ? 4 * G * HD : 32 * (HD + 8)) + G * attn_sc_ld(chunk_max) + 2 * G + 4;
+}
 
 template <int HD, int G>
 __device__ __forceinline__ void attn_partial_item(const u16* __restrict__ q, int64_t ldq, const u16* __restrict__ kc,
@@ -32,13 +47,20 @@ __device__ __forceinline__ void attn_partial_item(const u16* __restrict__ q, int
                                                   float* __restrict__ o_part, float* __restrict__ ml_part, int Hkv,
                                                   int Smax, int nsplit, int chunk_max, int split, int kvh, int b,
                                                   float* __restrict__ smem) {
+  static_assert(G <= 16, "the q heads of a kv head are the 16 columns of one matrix-core tile");
   constexpr int LPK = HD / 8;    // lanes that share one key row (8 elements each)
-  constexpr int KPW = 64 / LPK;  // keys per wave per iteration
-  float* qs = smem;                       // [G][HD]
-  float* ored = qs + G * HD;              // [4][G][HD]
-  float* sc = ored + 4 * G * HD;          // [G][chunk_max]
-  float* s_m = sc + G * chunk_max;        // [G]
-  float* s_l = s_m + G;                   // [G]
+  constexpr int KPW = 64 / LPK;  // keys per wave instruction
+  constexpr int NI = 16 / KPW;   // instructions per 16-key tile
+  constexpr int KS = HD / 32;    // matrix-core k-steps per row
+  constexpr int TPW = ATT_CHUNK / 64;  // tiles per wave
+  constexpr int LROW = HD + 8;   // LDS row length of the K piece, in elements
+  constexpr int REGION = 4 * G * HD > 32 * LROW ? 4 * G * HD : 32 * LROW;
+  float* ored = smem;                         // [4][G][HD]   (after the scores)
+  u16* kpiece = reinterpret_cast<u16*>(smem);  // [4 waves][16][LROW] bf16 (during the scores)
+  float* sc = smem + REGION;                  // [G][ldsc]
+  const int ldsc = attn_sc_ld(chunk_max);
+  float* s_m = sc + G * ldsc;                 // [G]
+  float* s_l = s_m + G;                       // [G]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int Hq = Hkv * G;
@@ -47,7 +69,7 @@ __device__ __forceinline__ void attn_partial_item(const u16* __restrict__ q, int
   const int chunk = (nkeys + nsplit - 1) / nsplit;
   const int k0 = split * chunk;
   const int k1 = k0 + chunk < nkeys ? k0 + chunk : nkeys;
-  const int n = k1 - k0;  // <= chunk_max by construction
+  const int n = k1 - k0;  // <= chunk_max <= ATT_CHUNK by construction
 
   float* o_out = o_part + (((int64_t)b * Hq + kvh * G) * nsplit + split) * HD;  // + g * nsplit * HD
   float* ml_out = ml_part + (((int64_t)b * Hq + kvh * G) * nsplit + split) * 2;  // + g * nsplit * 2
@@ -64,51 +86,54 @@ __device__ __forceinline__ void attn_partial_item(const u16* __restrict__ q, int
   const u16* kbase = kc + ((int64_t)b * Hkv + kvh) * Smax * HD;
   const u16* vbase = vc + ((int64_t)b * Hkv + kvh) * Smax * HD;
   const float scale = rsqrtf((float)HD);
-  // Keys are walked PFB iterations at a time with all loads of a batch requested together, and the
-  // first batch of K and of V is requested before anything else: a 64-key chunk (the usual size)
-  // then costs one memory round trip instead of one per iteration and per operand.
-  constexpr int PFB = 4;
-  const int key00 = k0 + wave * KPW + kl;
-  uint4 kfirst[PFB], vfirst[PFB];
+  // wave w owns the 16-key tiles w, w + 4, ...; instruction i of a tile covers keys i * KPW .. + KPW
+  uint4 kr[TPW][NI], vr[TPW][NI];
 #pragma unroll
-  for (int u = 0; u < PFB; ++u) {
-    const int key = key00 + u * 4 * KPW;
-    kfirst[u] = key < k1 ? ld16(kbase + (int64_t)key * HD + dl) : make_uint4(0, 0, 0, 0);
-    vfirst[u] = key < k1 ? ld16(vbase + (int64_t)key * HD + dl) : make_uint4(0, 0, 0, 0);
+  for (int j = 0; j < TPW; ++j)
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int key = k0 + (j * 4 + wave) * 16 + i * KPW + kl;
+      kr[j][i] = key < k1 ? ld16(kbase + (int64_t)key * HD + dl) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+  for (int j = 0; j < TPW; ++j)
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int key = k0 + (j * 4 + wave) * 16 + i * KPW + kl;
+      vr[j][i] = key < k1 ? ld16(vbase + (int64_t)key * HD + dl) : make_uint4(0, 0, 0, 0);
+    }
+  // q as B fragments: column = head lane % 16, k-step ks holds elements ks * 32 + (lane / 16) * 8 .. + 8
+  const int l16 = lane & 15, l4 = lane >> 4;
+  bf16x8_t qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const uint4 v = l16 < G ? ld16(q + (int64_t)b * ldq + (kvh * G + l16) * HD + ks * 32 + l4 * 8) : make_uint4(0, 0, 0, 0);
+    const u32x4_t vv = {v.x, v.y, v.z, v.w};
+    qf[ks] = __builtin_bit_cast(bf16x8_t, vv);
   }
-  for (int i = tid; i < G * HD; i += 256)
-    qs[i] = bf_to_f(q[(int64_t)b * ldq + (kvh * G + i / HD) * HD + (i % HD)]);
-  __syncthreads();
 
-  // ---- scores
+  // ---- scores: S[key][head] = sum_d K[key][d] q[head][d] on the matrix cores
   {
-    float qf[G][8];
+    u16* my = kpiece + wave * 16 * LROW;
 #pragma unroll
-    for (int g = 0; g < G; ++g)
+    for (int j = 0; j < TPW; ++j) {
+      const int t16 = (j * 4 + wave) * 16;  // first key of the tile, relative to k0
+      if (t16 < n) {  // uniform
+        asm volatile("" ::: "memory");
 #pragma unroll
-      for (int j = 0; j < 8; ++j) qf[g][j] = qs[g * HD + dl + j];
-    for (int kb = key00; kb < k1 + kl; kb += PFB * 4 * KPW) {  // "+ kl": keep the wave converged
-      uint4 kr[PFB];
+        for (int i = 0; i < NI; ++i) st16(my + (i * KPW + kl) * LROW + dl, kr[j][i]);
+        asm volatile("" ::: "memory");
+        f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-      for (int u = 0; u < PFB; ++u) {
-        const int key = kb + u * 4 * KPW;
-        kr[u] = kb == key00 ? kfirst[u] : (key < k1 ? ld16(kbase + (int64_t)key * HD + dl) : make_uint4(0, 0, 0, 0));
-      }
-#pragma unroll
-      for (int u = 0; u < PFB; ++u) {
-        const int key = kb + u * 4 * KPW;
-        const bool live = key < k1;
-        float kf[8];
-        unpack8(kr[u], kf);
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-          float s = 0.0f;
-#pragma unroll
-          for (int j = 0; j < 8; ++j) s = fmaf(kf[j], qf[g][j], s);
-#pragma unroll
-          for (int o = 1; o < LPK; o <<= 1) s += __shfl_xor(s, o, LR_WAVE);
-          if (live && (lane % LPK) == 0) sc[g * chunk_max + key - k0] = s * scale;
+        for (int ks = 0; ks < KS; ++ks) {
+          const bf16x8_t af = *reinterpret_cast<const bf16x8_t*>(my + l16 * LROW + ks * 32 + l4 * 8);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, qf[ks], acc, 0, 0, 0);
         }
+        asm volatile("" ::: "memory");
+        // accumulator element e: key t16 + 4 (lane / 16) + e, head lane % 16 (keys beyond n: never read)
+        if (l16 < G)
+          *reinterpret_cast<float4*>(sc + l16 * ldsc + t16 + 4 * l4) =
+              make_float4(acc[0] * scale, acc[1] * scale, acc[2] * scale, acc[3] * scale);
       }
     }
   }
@@ -117,12 +142,12 @@ __device__ __forceinline__ void attn_partial_item(const u16* __restrict__ q, int
   // ---- softmax statistics per head; sc becomes exp(s - max)
   for (int g = wave; g < G; g += 4) {
     float m = -INFINITY;
-    for (int i = lane; i < n; i += 64) m = fmaxf(m, sc[g * chunk_max + i]);
+    for (int i = lane; i < n; i += 64) m = fmaxf(m, sc[g * ldsc + i]);
     m = wave_max(m);
     float l = 0.0f;
     for (int i = lane; i < n; i += 64) {
-      const float p = expf(sc[g * chunk_max + i] - m);
-      sc[g * chunk_max + i] = p;
+      const float p = expf(sc[g * ldsc + i] - m);
+      sc[g * ldsc + i] = p;
       l += p;
     }
     l = wave_sum(l);
@@ -137,24 +162,22 @@ __device__ __forceinline__ void attn_partial_item(const u16* __restrict__ q, int
     for (int g = 0; g < G; ++g)
 #pragma unroll
       for (int j = 0; j < 8; ++j) acc[g][j] = 0.0f;
-    for (int kb = key00; kb < k1; kb += PFB * 4 * KPW) {
-      uint4 vr[PFB];
 #pragma unroll
-      for (int u = 0; u < PFB; ++u) {
-        const int key = kb + u * 4 * KPW;
-        vr[u] = kb == key00 ? vfirst[u] : (key < k1 ? ld16(vbase + (int64_t)key * HD + dl) : make_uint4(0, 0, 0, 0));
-      }
+    for (int j = 0; j < TPW; ++j) {
+      const int t16 = (j * 4 + wave) * 16;
+      if (t16 < n) {  // uniform
 #pragma unroll
-      for (int u = 0; u < PFB; ++u) {
-        const int key = kb + u * 4 * KPW;
-        if (key < k1) {
-          float vf[8];
-          unpack8(vr[u], vf);
+        for (int i = 0; i < NI; ++i) {
+          const int kk = t16 + i * KPW + kl;  // relative to k0
+          if (kk < n) {
+            float vf[8];
+            unpack8(vr[j][i], vf);
 #pragma unroll
-          for (int g = 0; g < G; ++g) {
-            const float p = sc[g * chunk_max + key - k0];
+            for (int g = 0; g < G; ++g) {
+              const float p = sc[g * ldsc + kk];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) acc[g][j] = fmaf(p, vf[j], acc[g][j]);
+              for (int e = 0; e < 8; ++e) acc[g][e] = fmaf(p, vf[e], acc[g][e]);
+            }
           }
         }
       }

@@ -164,7 +164,7 @@ class GPTBase(nn.Module):
     # -- shared pieces of the block schedules -----------------------------------------------------
     def _attention(self, ws: Workspace, blk, pos: Tensor, wqkv: nn.Module, out: Tensor):
         """ws.xn -> fused projection -> RoPE + cache write -> attention -> wo -> out (partial sum).
-        wqkv None: ws.qkv already holds the projection."""
+        wqkv None: ws.qkv already holds the projection.  out None: stop at the attention output ws.y."""
         cfg = self.config
         B, S = ws.B, ws.S
         Hq, Hkv, hd = cfg.n_head_local, cfg.n_kv_local, cfg.head_dim
@@ -176,7 +176,8 @@ class GPTBase(nn.Module):
             _hip.attn_decode(ws.qkv, kc, vc, pos, ws.y, ws.scratch, B, Hq, Hkv, hd)
         else:
             _hip.attn_prefill(ws.qkv, kc, vc, pos, ws.y, B, S, Hq, Hkv, hd)
-        _hip.module_linear(ws.y, blk.attention.wo, out)
+        if out is not None:
+            _hip.module_linear(ws.y, blk.attention.wo, out)
 
     def _mlp(self, ws: Workspace, blk, out: Tensor, xn: Optional[Tensor] = None):
         ff = blk.feed_forward

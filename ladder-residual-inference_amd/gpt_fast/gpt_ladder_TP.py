@@ -136,7 +136,8 @@ class GPTLadder(GPTBase):
                 side = self._side_stream = torch.cuda.Stream(device=main.device)
         pending_a = pending_m = None
         # decode batches of 5 to 64 rows on bf16 weights: the block's two input projections share one launch of
-        # the weight-streaming kernel (q/k/v next to up/gate, the latter storing silu(gate) * up directly)
+        # the weight-streaming kernel (q/k/v next to up/gate, the latter storing silu(gate) * up directly), and so
+        # do its two output projections (wo next to w2)
         multi = side is None and 4 < ws.B <= 64 and not hasattr(self.layers[0].attention.wqkv, "scales")
         for blk in self.layers:
             _hip.ladder_norms(ws.x, pending_a, pending_m, blk.attention_norm.weight, blk.ffn_norm.weight, ws.x, ws.xn,
@@ -144,8 +145,9 @@ class GPTLadder(GPTBase):
             if multi:
                 _hip.linear_multi((ws.xn, blk.attention.wqkv.weight, ws.qkv, _hip.EPI_NONE),
                                   (ws.xn2, blk.feed_forward.w1.weight, ws.act, _hip.EPI_SWIGLU))
-                self._attention(ws, blk, pos, None, ws.a)
-                _hip.linear(ws.act, blk.feed_forward.w2.weight, ws.m)
+                self._attention(ws, blk, pos, None, None)
+                _hip.linear_multi((ws.y, blk.attention.wo.weight, ws.a, _hip.EPI_NONE),
+                                  (ws.act, blk.feed_forward.w2.weight, ws.m, _hip.EPI_NONE))
             elif side is not None:
                 side.wait_stream(main)
                 with torch.cuda.stream(side):
