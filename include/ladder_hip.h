@@ -116,7 +116,20 @@ int lr_linear_tuned(const void* x, int64_t ldx, const void* w, void* y, int64_t 
  * feed_forward.w1), y[M, I] = bf16( bf16(silu(g)) * u ) with u, g the bf16-rounded projections
  * (LR_EPI_SWIGLU: utils.py:145-148 without the [M, 2 I] round trip).  Sums are fp32, added in a
  * fixed order.  The reference has no such call; it is what its compiled decode graph amounts to. */
-enum { LR_EPI_NONE = 0, LR_EPI_SWIGLU = 1 };
+enum { LR_EPI_NONE = 0, LR_EPI_SWIGLU = 1, LR_EPI_ROPE_KV = 2 };
+/* LR_EPI_ROPE_KV: the projection is the fused q/k/v projection of a DECODE step (one token per
+ * sequence, input row m = sequence m, N = (n_head + 2 n_kv_head) * head_dim) and finishes with what
+ * lr_rope_kv_write does to its output: q rotated in y, rotated k and v stored at slot pos[0] of the
+ * caches (utils.py:193-198, :50-59), bit for bit.  A position outside the cache or the table sets
+ * *err = LR_DEV_POS_RANGE and leaves the plain projection in y. */
+typedef struct lr_rope_kv {
+  const void* table;  /* freqs_cis [block_size, head_dim / 2, 2] */
+  const int32_t* pos; /* device: the position of this step */
+  void* k_cache;      /* [B, n_kv_head, smax, head_dim] */
+  void* v_cache;
+  int32_t* err;       /* device error word, may be NULL */
+  int32_t n_head, n_kv_head, head_dim, smax, block_size;
+} lr_rope_kv_t;
 typedef struct lr_projection {
   const void* x; /* [M, K] bf16, row stride ldx */
   int64_t ldx;
@@ -125,6 +138,7 @@ typedef struct lr_projection {
   int64_t ldy;
   int32_t N, K;
   int32_t epilogue;
+  const lr_rope_kv_t* rope; /* LR_EPI_ROPE_KV only, else ignored; read during the call */
 } lr_projection_t;
 int lr_linear_multi(const lr_projection_t* projections, int n_projections, int M, lr_stream_t stream);
 

@@ -321,7 +321,7 @@ extern "C" int lr_linear_tuned(const void* x, int64_t ldx, const void* w, void* 
   if (!act_swiglu && M <= 64) {
     // decode batches: the weight-streaming matrix-core kernel (stream_gemm.hip); shapes it declines fall through
     lr_projection_t pr;
-    pr.x = x; pr.ldx = ldx; pr.w = w; pr.y = y; pr.ldy = ldy; pr.N = N; pr.K = K; pr.epilogue = LR_EPI_NONE;
+    pr.x = x; pr.ldx = ldx; pr.w = w; pr.y = y; pr.ldy = ldy; pr.N = N; pr.K = K; pr.epilogue = LR_EPI_NONE; pr.rope = nullptr;
     const int rc = lr_linear_multi(&pr, 1, M, stream);
     if (rc != LR_E_UNSUPPORTED) return rc;
   }

@@ -18,7 +18,8 @@
 //
 // Two projections that read the same layer input can share one launch (the band index selects the
 // projection), and a projection whose weight holds [up; gate] rows can take the band as row PAIRS
-// and store bf16(bf16(silu(g)) * u) instead of u and g.
+// and store bf16(bf16(silu(g)) * u) instead of u and g.  The fused q/k/v projection of a decode step
+// can rotate q and k and put k and v into the cache on its way out (what lr_rope_kv_write does).
 #include "lr_common.h"
 
 namespace {
@@ -41,6 +42,12 @@ struct Proj {
   int rpw;       // rows (row pairs if pair_off) per workgroup
   int pair_off;  // 0, or the distance from an up row to its gate row (= outputs)
   int nwg;       // workgroups of this projection
+  // RoPE + KV-cache epilogue of a fused q/k/v projection (rope_table == nullptr: none)
+  const u16* rope_table;
+  const int32_t* pos;
+  u16 *k_cache, *v_cache;
+  int32_t* err;
+  int Hq, Hkv, hd, Smax, block_size;
 };
 
 template <int MT, int UNITS>
@@ -57,6 +64,7 @@ __global__ __launch_bounds__(NWV * 64) void k_stream_gemm(const Proj p0, const P
   const int64_t ldx = second ? p1.ldx : p0.ldx, ldy = second ? p1.ldy : p0.ldy;
   const int N = second ? p1.N : p0.N, K = second ? p1.K : p0.K, rpw = second ? p1.rpw : p0.rpw;
   const int pair_off = second ? p1.pair_off : p0.pair_off;
+  const u16* const rope_table = second ? p1.rope_table : p0.rope_table;
   const int band = second ? (int)blockIdx.x - p0.nwg : (int)blockIdx.x;
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -165,6 +173,47 @@ __global__ __launch_bounds__(NWV * 64) void k_stream_gemm(const Proj p0, const P
       for (int e = 0; e < 4; ++e) red[wave * WSTRIDE + ((u * MTILES + mt) * 4 + e) * 64 + lane] = acc[u][mt][e];
   __syncthreads();
   const int rows_out = pair_off ? 16 : 16 * UNITS;
+  if (rope_table != nullptr) {
+    // The fused q/k/v projection of a decode step (one token per sequence: input row m is sequence m):
+    // what lr_rope_kv_write would do to the stored row, done here on the (even, odd) output pairs.  A
+    // position outside the cache or the table: the plain projection is stored, the error word is set.
+    const Proj& pp = second ? p1 : p0;
+    const int hd = pp.hd, nq = pp.Hq * hd, nkv = pp.Hkv * hd;
+    const int ps = pp.pos[0];
+    const bool in_range = ps >= 0 && ps < pp.Smax && ps < pp.block_size;
+    if (!in_range && pp.err && band == 0 && tid == 0) *pp.err = LR_DEV_POS_RANGE;
+    for (int o = tid; o < (rows_out / 2) * MT; o += NWV * 64) {
+      const int r = 2 * (o % (rows_out / 2)), m = o / (rows_out / 2);
+      if (r >= nrows || m >= M) continue;
+      const int mt = m >> 4, ln = ((r & 15) >> 2) * 16 + (m & 15), e = r & 3, u = r >> 4;
+      float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+      for (int wv = 0; wv < NWV; ++wv) {
+        s0 += red[wv * WSTRIDE + ((u * MTILES + mt) * 4 + e) * 64 + ln];
+        s1 += red[wv * WSTRIDE + ((u * MTILES + mt) * 4 + e + 1) * 64 + ln];
+      }
+      const float x0 = round_bf(s0), x1 = round_bf(s1);
+      const int n = n0 + r;
+      u32 plain = pack_bf2(x0, x1), out = plain;
+      if (in_range) {
+        const int sect = n < nq ? 0 : (n < nq + nkv ? 1 : 2);
+        const int cc = n - (sect == 0 ? 0 : (sect == 1 ? nq : nq + nkv));
+        const int h = cc / hd, d = cc - h * hd;
+        if (sect < 2) {
+#pragma clang fp contract(off)
+          const u32 cs = *reinterpret_cast<const u32*>(rope_table + (int64_t)ps * hd + d);
+          const float c = bf_lo(cs), sn = bf_hi(cs);
+          const float a = x0 * c, b = x1 * sn, dd = x1 * c, ee = x0 * sn;
+          out = pack_bf2(a - b, dd + ee);
+        }
+        if (sect == 0) plain = out;  // q is rotated in place; k and v stay as projected, the cache gets them
+        if (sect == 1) *reinterpret_cast<u32*>(pp.k_cache + (((int64_t)m * pp.Hkv + h) * pp.Smax + ps) * hd + d) = out;
+        if (sect == 2) *reinterpret_cast<u32*>(pp.v_cache + (((int64_t)m * pp.Hkv + h) * pp.Smax + ps) * hd + d) = plain;
+      }
+      *reinterpret_cast<u32*>(yg + (int64_t)m * ldy + n) = plain;
+    }
+    return;
+  }
   for (int o = tid; o < rows_out * MT; o += NWV * 64) {
     const int r = o % rows_out, m = o / rows_out;
     if (r >= nrows || m >= M) continue;
@@ -199,11 +248,13 @@ static int num_cus() {
 // workgroup; with few weight rows and many input rows a band is not made thinner than `floor_rows`
 // (every band re-reads all input rows from L2).
 static void plan(Proj& p, int M, int cap, int ncu) {
+  // (the RoPE epilogue works on output pairs: bands of an even number of rows)
   const int items = p.pair_off ? p.pair_off : p.N;
   const int rounds = (items + ncu * cap - 1) / (ncu * cap);
   int rpw = (items + ncu * rounds - 1) / (ncu * rounds);
   const int floor_rows = M > 32 ? 16 : (M > 16 ? 8 : 4);
   if (rpw < floor_rows) rpw = floor_rows;
+  if (p.rope_table) rpw = (rpw + 1) & ~1;
   if (rpw > cap) rpw = cap;
   p.rpw = rpw;
   p.nwg = (items + rpw - 1) / rpw;
@@ -230,7 +281,7 @@ extern "C" int lr_linear_multi(const lr_projection_t* proj, int n_proj, int M, l
     LR_REQUIRE_PTR(q.w);
     LR_REQUIRE_PTR(q.y);
     if (q.N <= 0 || q.K <= 0 || q.ldx < q.K) return LR_E_SHAPE;
-    if (q.epilogue != LR_EPI_NONE && q.epilogue != LR_EPI_SWIGLU) return LR_E_SHAPE;
+    if (q.epilogue != LR_EPI_NONE && q.epilogue != LR_EPI_SWIGLU && q.epilogue != LR_EPI_ROPE_KV) return LR_E_SHAPE;
     const bool pair = q.epilogue == LR_EPI_SWIGLU;
     if (pair && q.N % 2) return LR_E_SHAPE;
     if (q.ldy < (pair ? q.N / 2 : q.N)) return LR_E_SHAPE;
@@ -243,6 +294,20 @@ extern "C" int lr_linear_multi(const lr_projection_t* proj, int n_proj, int M, l
     p.ldx = q.ldx; p.ldy = q.ldy; p.N = q.N; p.K = q.K;
     p.pair_off = pair ? q.N / 2 : 0;
     any_pair = any_pair || pair;
+    if (q.epilogue == LR_EPI_ROPE_KV) {
+      const lr_rope_kv_t* r = q.rope;
+      if (r == nullptr || r->pos == nullptr) return LR_E_NULL;
+      LR_REQUIRE_PTR(r->table);
+      LR_REQUIRE_PTR(r->k_cache);
+      LR_REQUIRE_PTR(r->v_cache);
+      if (r->n_head <= 0 || r->n_kv_head <= 0 || r->head_dim <= 0 || r->smax <= 0 || r->block_size <= 0 ||
+          (int64_t)(r->n_head + 2 * r->n_kv_head) * r->head_dim != q.N || q.ldy % 2)
+        return LR_E_SHAPE;
+      if (r->head_dim % 8) return LR_E_ALIGN;
+      p.rope_table = (const u16*)r->table; p.pos = r->pos; p.k_cache = (u16*)r->k_cache; p.v_cache = (u16*)r->v_cache;
+      p.err = r->err; p.Hq = r->n_head; p.Hkv = r->n_kv_head; p.hd = r->head_dim; p.Smax = r->smax;
+      p.block_size = r->block_size;
+    }
   }
   const int ncu = num_cus();
   if (ncu < 1) return LR_E_LAUNCH;

@@ -181,21 +181,44 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, act_swiglu: bool
 _FP8_SCRATCH = {}
 
 
+class _RopeKv(ctypes.Structure):   # lr_rope_kv_t
+    _fields_ = [("table", c_void_p), ("pos", c_void_p), ("k_cache", c_void_p), ("v_cache", c_void_p), ("err", c_void_p),
+                ("n_head", c_int32), ("n_kv_head", c_int32), ("head_dim", c_int32), ("smax", c_int32),
+                ("block_size", c_int32)]
+
+
 class _Projection(ctypes.Structure):   # lr_projection_t
     _fields_ = [("x", c_void_p), ("ldx", c_int64), ("w", c_void_p), ("y", c_void_p), ("ldy", c_int64),
-                ("N", ctypes.c_int32), ("K", ctypes.c_int32), ("epilogue", ctypes.c_int32)]
+                ("N", c_int32), ("K", c_int32), ("epilogue", c_int32), ("rope", ctypes.POINTER(_RopeKv))]
 
 
-EPI_NONE, EPI_SWIGLU = 0, 1
+EPI_NONE, EPI_SWIGLU, EPI_ROPE_KV = 0, 1, 2
+
+
+def rope_kv_epilogue(table, pos, k_cache, v_cache, Hq, Hkv, hd):
+    """The descriptor an EPI_ROPE_KV projection of linear_multi carries (decode: one token per sequence)."""
+    assert pos.dtype == torch.int32 and pos.is_cuda and pos.numel() == 1
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape == v_cache.shape
+    _, hkv_c, Smax, hd_c = k_cache.shape
+    assert hkv_c == Hkv and hd_c == hd and table.is_contiguous() and table.shape[-2:] == (hd // 2, 2)
+    return _RopeKv(_dev(table), pos.data_ptr(), _dev(k_cache), _dev(v_cache),
+                   device_error_word(k_cache.device).data_ptr(), Hq, Hkv, hd, Smax, table.shape[0])
 
 
 def linear_multi(*projections):
     """One launch of the weight-streaming kernel for one or two projections of the same M <= 64 rows.
     Each projection is (x [M, K], w [N, K], out, epilogue): EPI_NONE -> out [M, N] = x @ w^T;
-    EPI_SWIGLU -> w holds [up; gate] rows and out [M, N / 2] = silu(gate) * up (lr_linear_multi)."""
+    EPI_SWIGLU -> w holds [up; gate] rows and out [M, N / 2] = silu(gate) * up; or, for the fused q/k/v
+    projection of a decode step, (x, w, out, rope_kv_epilogue(...)): q rotated in out, k and v into the cache
+    (lr_linear_multi)."""
     arr = (_Projection * len(projections))()
     M = None
+    keep = []
     for i, (x, w, out, epi) in enumerate(projections):
+        rope = None
+        if isinstance(epi, _RopeKv):
+            rope, epi = epi, EPI_ROPE_KV
+            keep.append(rope)
         m, K, ldx = _rows_ld(x)
         N, Kw = w.shape
         Mo, No, ldy = _rows_ld(out)
@@ -203,7 +226,8 @@ def linear_multi(*projections):
             (x.shape, w.shape, out.shape, epi)
         assert M is None or M == m
         M = m
-        arr[i] = _Projection(_dev(x), ldx, _dev(w), _dev(out), ldy, N, K, epi)
+        arr[i] = _Projection(_dev(x), ldx, _dev(w), _dev(out), ldy, N, K, epi,
+                             ctypes.pointer(rope) if rope is not None else None)
     _check(load().lr_linear_multi(ctypes.cast(arr, c_void_p), len(projections), M, _stream()), "lr_linear_multi")
 
 

@@ -162,16 +162,18 @@ class GPTBase(nn.Module):
         raise NotImplementedError
 
     # -- shared pieces of the block schedules -----------------------------------------------------
-    def _attention(self, ws: Workspace, blk, pos: Tensor, wqkv: nn.Module, out: Tensor):
+    def _attention(self, ws: Workspace, blk, pos: Tensor, wqkv: nn.Module, out: Tensor, roped: bool = False):
         """ws.xn -> fused projection -> RoPE + cache write -> attention -> wo -> out (partial sum).
-        wqkv None: ws.qkv already holds the projection.  out None: stop at the attention output ws.y."""
+        wqkv None: ws.qkv already holds the projection (roped: rotated, with k and v already in the cache).
+        out None: stop at the attention output ws.y."""
         cfg = self.config
         B, S = ws.B, ws.S
         Hq, Hkv, hd = cfg.n_head_local, cfg.n_kv_local, cfg.head_dim
         kc, vc = blk.attention.kv_cache.k_cache, blk.attention.kv_cache.v_cache
         if wqkv is not None:
             _hip.module_linear(ws.xn, wqkv, ws.qkv)
-        _hip.rope_kv_write(ws.qkv, self.freqs_cis, False, pos, kc, vc, B, S, Hq, Hkv, hd)
+        if not roped:
+            _hip.rope_kv_write(ws.qkv, self.freqs_cis, False, pos, kc, vc, B, S, Hq, Hkv, hd)
         if S == 1:
             _hip.attn_decode(ws.qkv, kc, vc, pos, ws.y, ws.scratch, B, Hq, Hkv, hd)
         else:

@@ -127,7 +127,8 @@ class GPTLadder(GPTBase):
         attention output), then the attention chain (wqkv, RoPE + cache write, attention, wo) and the MLP chain
         (w1, SwiGLU, w2) -- one after the other, or on two streams where the reference overlaps an all-reduce with
         the next module (gpt_ladder_TP.py:339-349)."""
-        eps = self.config.norm_eps
+        cfg = self.config
+        eps = cfg.norm_eps
         main = side = None
         if self.overlap_modules:
             main = torch.cuda.current_stream()
@@ -136,16 +137,19 @@ class GPTLadder(GPTBase):
                 side = self._side_stream = torch.cuda.Stream(device=main.device)
         pending_a = pending_m = None
         # decode batches of 5 to 64 rows on bf16 weights: the block's two input projections share one launch of
-        # the weight-streaming kernel (q/k/v next to up/gate, the latter storing silu(gate) * up directly), and so
-        # do its two output projections (wo next to w2)
+        # the weight-streaming kernel (q/k/v -- rotated and cached on the way out -- next to up/gate, which stores
+        # silu(gate) * up directly), and so do its two output projections (wo next to w2)
         multi = side is None and 4 < ws.B <= 64 and not hasattr(self.layers[0].attention.wqkv, "scales")
         for blk in self.layers:
             _hip.ladder_norms(ws.x, pending_a, pending_m, blk.attention_norm.weight, blk.ffn_norm.weight, ws.x, ws.xn,
                               ws.xn2, eps)
             if multi:
-                _hip.linear_multi((ws.xn, blk.attention.wqkv.weight, ws.qkv, _hip.EPI_NONE),
+                kv = blk.attention.kv_cache
+                rope = _hip.rope_kv_epilogue(self.freqs_cis, pos, kv.k_cache, kv.v_cache, cfg.n_head_local,
+                                             cfg.n_kv_local, cfg.head_dim)
+                _hip.linear_multi((ws.xn, blk.attention.wqkv.weight, ws.qkv, rope),
                                   (ws.xn2, blk.feed_forward.w1.weight, ws.act, _hip.EPI_SWIGLU))
-                self._attention(ws, blk, pos, None, None)
+                self._attention(ws, blk, pos, None, None, roped=True)
                 _hip.linear_multi((ws.y, blk.attention.wo.weight, ws.a, _hip.EPI_NONE),
                                   (ws.act, blk.feed_forward.w2.weight, ws.m, _hip.EPI_NONE))
             elif side is not None:

@@ -205,6 +205,52 @@ def test_linear_multi_swiglu_epilogue_equals_the_two_step_path(hip):
     assert torch.equal(act, two_step)
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,hd,D", [(8, 8, 1, 128, 1024), (64, 8, 1, 128, 512), (16, 32, 8, 128, 264),
+                                            (5, 4, 2, 64, 136), (1, 2, 2, 64, 64)])
+@pytest.mark.parametrize("pos_value", [0, 37])
+def test_linear_multi_rope_kv_epilogue_equals_projection_then_rope_kv_write(hip, B, Hq, Hkv, hd, D, pos_value):
+    """The q/k/v projection that rotates and caches on its way out leaves q, the K slot and the V slot exactly as
+    the plain projection followed by lr_rope_kv_write does, and touches no other cache slot."""
+    Smax, block = 48, 64
+    N = (Hq + 2 * Hkv) * hd
+    x, w = rnd(B, D, seed=40), rnd(N, D, seed=41, scale=0.05)
+    table = O.rope_table(block, hd, 10000.0, BF).to(DEV)
+    pos = torch.tensor([pos_value], dtype=torch.int32, device=DEV)
+    kc = [rnd(B, Hkv, Smax, hd, seed=42) for _ in range(2)]
+    vc = [rnd(B, Hkv, Smax, hd, seed=43) for _ in range(2)]
+    # reference path
+    q_ref = torch.empty(B, N, dtype=BF, device=DEV)
+    hip.linear_multi((x, w, q_ref, hip.EPI_NONE))
+    k_proj = q_ref[:, Hq * hd:].clone()
+    hip.rope_kv_write(q_ref, table, False, pos, kc[0], vc[0], B, 1, Hq, Hkv, hd)
+    # fused path
+    q = torch.empty(B, N, dtype=BF, device=DEV)
+    hip.linear_multi((x, w, q, hip.rope_kv_epilogue(table, pos, kc[1], vc[1], Hq, Hkv, hd)))
+    assert torch.equal(q[:, :Hq * hd], q_ref[:, :Hq * hd])
+    assert torch.equal(q[:, Hq * hd:], k_proj)          # k and v stay as projected in the row buffer
+    assert torch.equal(kc[1], kc[0]) and torch.equal(vc[1], vc[0])
+    assert not torch.equal(kc[1][:, :, pos_value], rnd(B, Hkv, Smax, hd, seed=42)[:, :, pos_value])
+
+
+def test_linear_multi_rope_kv_epilogue_reports_a_position_outside_the_cache(hip):
+    B, Hq, Hkv, hd, D, Smax = 8, 4, 1, 64, 128, 16
+    N = (Hq + 2 * Hkv) * hd
+    x, w = rnd(B, D, seed=44), rnd(N, D, seed=45, scale=0.05)
+    table = O.rope_table(32, hd, 10000.0, BF).to(DEV)
+    kc, vc = rnd(B, Hkv, Smax, hd, seed=46), rnd(B, Hkv, Smax, hd, seed=47)
+    kc0, vc0 = kc.clone(), vc.clone()
+    err = hip.device_error_word(DEV)
+    err.zero_()
+    plain, q = torch.empty(B, N, dtype=BF, device=DEV), torch.empty(B, N, dtype=BF, device=DEV)
+    hip.linear_multi((x, w, plain, hip.EPI_NONE))
+    hip.linear_multi((x, w, q, hip.rope_kv_epilogue(table, torch.tensor([Smax], dtype=torch.int32, device=DEV), kc, vc,
+                                                    Hq, Hkv, hd)))
+    torch.cuda.synchronize()
+    assert int(err.item()) == hip.DEV_POS_RANGE
+    err.zero_()
+    assert torch.equal(q, plain) and torch.equal(kc, kc0) and torch.equal(vc, vc0)
+
+
 def test_linear_multi_is_deterministic(hip):
     x, w = rnd(64, 8192, seed=36), rnd(1280, 8192, seed=37, scale=0.02)
     ys = []
