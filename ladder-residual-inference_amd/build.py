@@ -15,6 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "gpt_fast", "libladder_hip.so")
+PROF_LIB = os.path.join(HERE, "gpt_fast", "libladder_hip_prof.so")
 HEADERS = [os.path.join(CSRC, h) for h in ("lr_common.h", "attn_decode_item.h")] + \
     [os.path.join(HERE, "..", "include", "ladder_hip.h")]
 
@@ -33,11 +34,11 @@ def _stale(target, deps):
     return any(os.path.getmtime(d) > t for d in deps)
 
 
-def _compile(src, force):
-    obj = os.path.join(OBJ, os.path.basename(src).replace(".hip", ".o"))
+def _compile(src, force, extra=(), suffix=""):
+    obj = os.path.join(OBJ, os.path.basename(src).replace(".hip", suffix + ".o"))
     if not force and not _stale(obj, [src] + HEADERS):
         return obj, False
-    cmd = ["hipcc"] + FLAGS + ["-c", src, "-o", obj]
+    cmd = ["hipcc"] + FLAGS + list(extra) + ["-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "is not a recognized feature for this target" not in l)
     if r.returncode != 0:
@@ -63,7 +64,29 @@ def build(force=False, verbose=True):
     return LIB
 
 
+def build_step_profile(force=False, verbose=True):
+    """A second library, gpt_fast/libladder_hip_prof.so, whose decode-step kernel records wall-clock stamps per
+    workgroup and phase (-DLR_STEP_PROFILE; read by step_phases.py).  The product library carries none of it."""
+    build(force=force, verbose=False)
+    obj, changed = _compile(os.path.join(CSRC, "ladder_step.hip"), force, ("-DLR_STEP_PROFILE",), "_prof")
+    objs = [os.path.join(OBJ, f) for f in sorted(os.listdir(OBJ))
+            if f.endswith(".o") and f not in ("ladder_step.o", "ladder_step_prof.o")] + [obj]
+    if force or changed or _stale(PROF_LIB, objs):
+        r = subprocess.run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PROF_LIB] + objs,
+                           capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("link failed:\n" + r.stderr)
+    if verbose:
+        print(f"built {PROF_LIB}")
+    return PROF_LIB
+
+
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--force", action="store_true")
-    build(force=ap.parse_args().force)
+    ap.add_argument("--profile-step", action="store_true",
+                    help="also build libladder_hip_prof.so (decode-step kernel with per-phase time stamps)")
+    args = ap.parse_args()
+    build(force=args.force)
+    if args.profile_step:
+        build_step_profile(force=args.force)

@@ -720,7 +720,7 @@ __device__ __forceinline__ void residual_step(const StepParams& p, const Coh& co
                                               bool has_d1, unsigned d1_wo, unsigned d1_tag, bool early1,
                                               const EarlyWords<M>& e1, bool has_d2, unsigned d2_wo, unsigned d2_tag,
                                               const u16* gain, u16* x, float* red, bool do_prime, const Job& first,
-                                              Pipe& pipe) {
+                                              Pipe& pipe, unsigned long long* stamp = nullptr) {
   const int tid = opaque_tid(), D = p.D;
   float ss[M];
   // the gain is needed only in pass 2 but is requested now: its latency hides behind pass 1
@@ -787,7 +787,9 @@ __device__ __forceinline__ void residual_step(const StepParams& p, const Coh& co
   // wave's loads return in order and a CU serves them at a bounded rate, so requested earlier they
   // would stand between this phase and the words it waits for; from here they travel while the
   // norm is finished.
+  if (stamp && tid == 0) stamp[13] = wall_clock64();
   if (do_prime) prime(first, tid & 63, pipe);
+  if (stamp && tid == 0) stamp[15] = wall_clock64();
   if (gain == nullptr) return;  // uniform: only the residual was wanted (each lane revisits its own elements later)
 #pragma unroll
   for (int m = 0; m < M; ++m) ss[m] = wave_sum(ss[m]);
@@ -796,6 +798,7 @@ __device__ __forceinline__ void residual_step(const StepParams& p, const Coh& co
     for (int m = 0; m < M; ++m) red[(tid >> 6) * M + m] = ss[m];
   }
   wg_sync();
+  if (stamp && tid == 0) stamp[14] = wall_clock64();
   // pass 2: scale in place (each lane revisits the elements it wrote)
 #pragma unroll
   for (int m = 0; m < M; ++m) {
@@ -1278,7 +1281,8 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
       Job j_first = j_head;
       if (!last) j_first = load_job(jtab, JK_QKV, wave, ring_ptr(lring, t + 1, LP_WQKV));
       residual_step<M>(p, coh, xr, nullptr, true, p.oa, tag, false, ew, last, p.om, tag,
-                       last ? p.final_norm : ring_ptr(lring, t + 1, LP_ATTN_NORM), xa, red, true, j_first, pipe);
+                       last ? p.final_norm : ring_ptr(lring, t + 1, LP_ATTN_NORM), xa, red, true, j_first, pipe,
+                       LR_STAMP_PTR);
     }
     LR_STAMP(0)
     {

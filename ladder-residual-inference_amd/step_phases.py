@@ -1,0 +1,94 @@
+"""Where the time of one decode step of the one-kernel Ladder path goes, per phase of a layer slot.
+
+    python build.py --profile-step          # once, anywhere hipcc runs: gpt_fast/libladder_hip_prof.so
+    python step_phases.py [--model gpt_ladder:ladder-70b-tp8] [--prompt 2048] [--slot 40]
+
+The profile build of the step kernel writes, per workgroup, a 100 MHz wall-clock stamp at every phase boundary of
+four consecutive layer slots (lr_ladder_step_profile, profile builds only).  This script runs a few steps of the
+benchmark workload (random weights, batch 1) on that library and prints, per phase, the mean / min / max duration
+over the workgroups -- attention workgroups and weight-streaming workgroups separately -- and the slot length."""
+import argparse
+import ctypes
+import os
+import sys
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, HERE)
+
+from gpt_fast import _hip  # noqa: E402
+
+PHASES = ["slot start", "(top of loop)", "wqkv rows", "R += m, ffn norm | R += m", "w1 rows + SwiGLU | attention + merge",
+          "wait for merged attention output", "wo rows", "wait for activations", "w2 rows"]
+ATT_PARTS = {"attention: q wait + RoPE": (3, 10), "attention: scores": (10, 11), "attention: softmax": (11, 12),
+             "attention: P.V + merge": (12, 4)}
+CLOSE_PARTS = {"closing R += a, norm: words + pass 1": (8, 13), "closing: first units of the next job": (13, 15),
+               "closing: sum of squares, barrier": (15, 14), "closing: pass 2": (14, 0)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--model", default="gpt_ladder:ladder-70b-tp8")
+    ap.add_argument("--prompt", type=int, default=2048)
+    ap.add_argument("--slot", type=int, default=40, help="first of the four layer slots that are stamped")
+    ap.add_argument("--steps", type=int, default=20)
+    args = ap.parse_args()
+
+    prof_lib = os.path.join(HERE, "gpt_fast", "libladder_hip_prof.so")
+    if not os.path.exists(prof_lib):
+        raise SystemExit(f"{prof_lib} is missing: python build.py --profile-step")
+    _hip._LIB_PATH = prof_lib
+    import benchmark as bm
+
+    model = bm._load_model(args.model, "cuda", torch.bfloat16, seed=0, verbose=False)
+    T = args.prompt
+    model.setup_caches(1, T + 64)
+    model.last_logits_only = True
+    lib = _hip.load()
+    lib.lr_ladder_step_profile.restype = ctypes.c_size_t
+    lib.lr_ladder_step_profile.argtypes = [ctypes.c_void_p, ctypes.c_int]
+    with torch.no_grad():
+        prompt = torch.randint(0, model.config.vocab_size, (T,), device="cuda")
+        first = bm.prefill(model, prompt.view(1, -1), torch.arange(T, device="cuda", dtype=torch.int32), greedy=True).clone()
+        pos = torch.tensor([T], dtype=torch.int32, device="cuda")
+        for _ in range(3):
+            model(first.view(1, 1), pos)
+        nbytes = lib.lr_ladder_step_profile(None, 0)
+        buf = torch.zeros(nbytes // 8, dtype=torch.int64, device="cuda")
+        lib.lr_ladder_step_profile(buf.data_ptr(), args.slot)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            model(first.view(1, 1), pos)
+        e1.record()
+        torch.cuda.synchronize()
+        lib.lr_ladder_step_profile(None, 0)
+    model.check_device_errors()
+    print(f"{args.model}, batch 1, position {T}: {e0.elapsed_time(e1) / args.steps:.3f} ms per step (profile build, eager launches)")
+    a = buf.cpu().numpy().reshape(-1, 4, 16).astype(np.float64) * 0.01   # [workgroup][slot][stamp] in microseconds
+    nwg = a.shape[0]
+    s = 1   # second of the four stamped slots
+    na = int((a[:, s, 10] > 0).sum())   # only attention workgroups write the attention stamps (the first `na`)
+    groups = {"weight-streaming workgroups": slice(na, nwg), "attention workgroups": slice(0, na)}
+    print(f"layer slot {args.slot + s}; {nwg} workgroups, {na} of them attention workgroups; durations in microseconds")
+    for gname, sl in groups.items():
+        print(f"  {gname}")
+        for k in range(2, len(PHASES)):
+            d = a[sl, s, k] - a[sl, s, k - 1]
+            print(f"    {PHASES[k]:42s} mean {d.mean():6.2f}  min {d.min():6.2f}  max {d.max():6.2f}")
+        for nm, (k0, k1) in CLOSE_PARTS.items():
+            d = a[sl, s, k1] - a[sl, s, k0]
+            print(f"    {nm:42s} mean {d.mean():6.2f}  min {d.min():6.2f}  max {d.max():6.2f}")
+    for nm, (k0, k1) in ATT_PARTS.items():
+        d = a[:na, s, k1] - a[:na, s, k0]
+        print(f"    {nm:42s} mean {d.mean():6.2f}  min {d.min():6.2f}  max {d.max():6.2f}")
+    lens = [(a[:, j + 1, 1] - a[:, j, 1]).mean() for j in range(3)]
+    print("  slot length (loop top to loop top), three consecutive slots: " + ", ".join(f"{x:.2f}" for x in lens))
+    ends = a[:, s, 8] - a[:, s, 1].min()
+    print(f"  w2 finish time after the first workgroup entered the slot: mean {ends.mean():.2f}, last {ends.max():.2f}")
+
+
+if __name__ == "__main__":
+    main()
