@@ -28,7 +28,8 @@ Prints ONE JSON line.  `value` = decoded tokens per second (whole job = the one 
                threads used (the process's CPU share: OMP_NUM_THREADS when set, else every core),
                `host_cpus` = os.cpu_count().
 Measured in the same run and reported as extra keys (not the headline; --no-extras skips them):
-`batched`     : the same rank shard at batch 8 and 64 (per-op kernels, hipGraph replay): ms per step,
+`batched`     : the same rank shard at batch 8 and 64, the 8B model at batch 16 (prompt 1024) and the 405B
+               rank shard at batch 16 (context 4096) -- per-op kernels, hipGraph replay: ms per step,
                tok/s, algorithmic GB/s and its fraction of 8 TB/s.
 `fp8`         : the same shard with weight-only e4m3 projections at batch 1 (per-op kernels): ms per
                step and the fraction of 8 TB/s on ITS algorithmic bytes (one byte per weight + scales).
@@ -116,11 +117,30 @@ def extra_batched(bm, model, prompt, T, batches=(8, 64), K=32, W=5):
         ms, _, dg = decode_run(bm, model, prompt, B, T, K, W)
         nbytes = sum(bm.decode_bytes_per_step(cfg, B, T + i) for i in range(K)) / K
         gbps = nbytes / (ms * 1e-3) / 1e9
-        out.append({"batch": B, "ms_per_step": round(ms, 4), "tok_per_s": round(B * 1e3 / ms, 1),
-                    "bytes_per_step": int(nbytes), "achieved_GBps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4),
-                    "steps": K})
+        out.append({"model": "gpt_ladder:ladder-70b-tp8", "batch": B, "prompt_len": T, "ms_per_step": round(ms, 4),
+                    "tok_per_s": round(B * 1e3 / ms, 1), "bytes_per_step": int(nbytes), "achieved_GBps": round(gbps, 1),
+                    "frac": round(gbps / HBM_PEAK_GBPS, 4), "steps": K})
         del dg
     return out
+
+
+def extra_model_decode(bm, name, B, T, K=16, W=3):
+    """Another decode configuration of the benchmark set, on a model of its own (random weights, per-op kernels)."""
+    import torch
+
+    model = bm._load_model(name, "cuda", torch.bfloat16, seed=0, verbose=False)
+    model.last_logits_only = True
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1)
+    prompt = torch.randint(0, model.config.vocab_size, (T,), device="cuda", generator=g)
+    ms, _, dg = decode_run(bm, model, prompt, B, T, K, W)
+    nbytes = sum(bm.decode_bytes_per_step(model.config, B, T + i) for i in range(K)) / K
+    gbps = nbytes / (ms * 1e-3) / 1e9
+    del dg, model
+    torch.cuda.empty_cache()
+    return {"model": name, "batch": B, "prompt_len": T, "ms_per_step": round(ms, 4), "tok_per_s": round(B * 1e3 / ms, 1),
+            "bytes_per_step": int(nbytes), "achieved_GBps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4),
+            "steps": K}
 
 
 def fp8_bytes_per_step(cfg, B, pos):
@@ -344,6 +364,9 @@ def main():
         del model
         torch.cuda.empty_cache()
         out["prefill"] = extra_prefill(bm)
+        # the other decode configurations of the benchmark set: the 8B model at batch 16, the 405B rank shard at batch 16
+        out["batched"].append(extra_model_decode(bm, "gpt_ladder:ladder-8b", 16, 1024))
+        out["batched"].append(extra_model_decode(bm, "gpt_ladder:ladder-405b-tp8", 16, 4096))
     else:
         del model
     torch.cuda.empty_cache()
