@@ -142,6 +142,16 @@ typedef struct lr_projection {
 } lr_projection_t;
 int lr_linear_multi(const lr_projection_t* projections, int n_projections, int M, lr_stream_t stream);
 
+/* The MLP's first projection with the activation applied on the way out (utils.py:145-148):
+ *     y[M, I] = bf16( bf16(silu(g)) * u ),  [u | g] = bf16(x w^T),  w [2 I, K] = [up; gate] rows, N = 2 I.
+ * M <= 64: lr_linear_multi's LR_EPI_SWIGLU; M >= 512 on a large enough grid: the 256 x 256 tile
+ * matrix-core GEMM on tiles of 128 row PAIRS (a lane holds both halves of a pair); otherwise the
+ * projection goes to `scratch` ([M, N] bf16, scratch_bytes >= 2 M N, then ldy must equal I) and
+ * lr_swiglu follows.  scratch may be NULL when one of the first two cases applies.  Same bits as
+ * lr_linear followed by lr_swiglu. */
+int lr_linear_swiglu_out(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
+                         void* scratch, size_t scratch_bytes, lr_stream_t stream);
+
 /* Weight-only fp8 linear:  y[m, n] = bf16( bf16( sum_k x[m, k] * w8[n, k] ) * scales[n] ).
  * w8 [N, K] dense float8 e4m3 (OCP "e4m3fn": bias 7, no infinities, max 448), one byte per weight;
  * scales [N] bf16, one per output row; x, y bf16 as in lr_linear.  K % 16 == 0.

@@ -139,7 +139,7 @@ constexpr int GM = 256, GN = 256;
 
 __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int64_t ldx, const u16* __restrict__ w,
                                                   u16* __restrict__ y, int64_t ldy, int M, int N, int K, int tm,
-                                                  int tn) {
+                                                  int tn, int pair_off) {
   extern __shared__ __attribute__((aligned(16))) u16 gsm[];
   u16* xs = gsm;                      // [2][GM * LDT]
   u16* ws = gsm + 2 * GM * LDT;       // [2][GN * LDT]
@@ -160,7 +160,10 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
       nt = id - mt * tn;
     }
   }
-  const int m0 = mt * GM, n0 = nt * GN;
+  // pair_off != 0: w holds [up; gate] rows (pair_off = number of pairs) and the tile covers 128 PAIRS: each wave's
+  // 128 weight rows are 64 up rows followed by the 64 gate rows of the same pairs, so that a lane ends up with
+  // both halves of a pair and stores bf16(bf16(silu(g)) * u) -- N is then the number of pairs
+  const int m0 = mt * GM, n0 = nt * (pair_off ? GN / 2 : GN);
 
   // staging assignment: 2048 16-byte chunks per operand tile, 8 per thread
   f32x16_t acc[4][4];
@@ -181,7 +184,13 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
   for (int i = 0; i < 8; ++i) {
     const int r = srow0 + i * 32;
     xoff[i] = m0 + r < M ? (int)((int64_t)r * ldx * 2) : (int)0x80000000;
-    woff[i] = n0 + r < N ? r * K * 2 : (int)0x80000000;
+    if (pair_off) {
+      const int wv = i >> 2, b = i & 3;                      // r = wv * 128 + b * 32 + srow0
+      const int pr = wv * 64 + (b & 1) * 32 + srow0;          // pair inside the tile
+      woff[i] = n0 + pr < N ? (int)((int64_t)((b >> 1) * pair_off + pr) * K * 2) : (int)0x80000000;
+    } else {
+      woff[i] = n0 + r < N ? r * K * 2 : (int)0x80000000;
+    }
   }
   auto fetch = [&](const __amdgpu_buffer_rsrc_t& res, int rowoff, int k) -> uint4 {
     const int off = (k < K && rowoff >= 0) ? rowoff + k * 2 : (int)0x80000000;
@@ -214,6 +223,13 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
   __syncthreads();
 
   const int arow = lane & 31, akq = (lane >> 5) * 8;
+  // Fragments of k-step ks + 1 are read from LDS while the matrix instructions of k-step ks run; those of the next
+  // tile's k-step 0 during this tile's last k-step, behind the one workgroup barrier of the iteration.
+  bf16x8_t af[2][4], bfr[2][4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a) af[0][a] = *reinterpret_cast<const bf16x8_t*>(&xs[(wm * 128 + a * 32 + arow) * LDT + akq]);
+#pragma unroll
+  for (int b = 0; b < 4; ++b) bfr[0][b] = *reinterpret_cast<const bf16x8_t*>(&ws[(wn * 128 + b * 32 + arow) * LDT + akq]);
   for (int kt = 0; kt < nk; ++kt) {
     const int cur = kt & 1;
     const u16* xc = xs + cur * GM * LDT;
@@ -221,51 +237,80 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
     u16* xn = xs + (cur ^ 1) * GM * LDT;
     u16* wn_ = ws + (cur ^ 1) * GN * LDT;
     const int k2 = (kt + 2) * BK;
-    // the fragments of k-step ks + 1 are read from LDS while the 16 MFMAs of k-step ks run
-    bf16x8_t af[2][4], bfr[2][4];
-#pragma unroll
-    for (int a = 0; a < 4; ++a)
-      af[0][a] = *reinterpret_cast<const bf16x8_t*>(&xc[(wm * 128 + a * 32 + arow) * LDT + akq]);
-#pragma unroll
-    for (int b = 0; b < 4; ++b)
-      bfr[0][b] = *reinterpret_cast<const bf16x8_t*>(&wc[(wn * 128 + b * 32 + arow) * LDT + akq]);
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
       const int c = ks & 1, nx = c ^ 1;
-      __builtin_amdgcn_sched_barrier(0);
-      if (ks + 1 < BK / 16) {
+      const bool last = ks + 1 == BK / 16;
+      // One non-matrix instruction in the shadow of every matrix instruction (a wave issues in order: grouped, the
+      // sixteen matrix instructions of a k-step would be followed by ~16 LDS / global instructions with the matrix
+      // pipe idle).  K-steps 0..2: the eight fragment reads of the next k-step, the four LDS writes of the staged
+      // quarter, the four global loads of the quarter after it.  Last k-step: the writes first, then the barrier
+      // (every wave has written the next tile and has read all it needs of this one), the loads, and the fragment
+      // reads of the NEXT tile's k-step 0 -- so that an iteration does not open with the matrix pipe waiting for LDS.
 #pragma unroll
-        for (int a = 0; a < 4; ++a)
-          af[nx][a] = *reinterpret_cast<const bf16x8_t*>(&xc[(wm * 128 + a * 32 + arow) * LDT + (ks + 1) * 16 + akq]);
-#pragma unroll
-        for (int b = 0; b < 4; ++b)
-          bfr[nx][b] = *reinterpret_cast<const bf16x8_t*>(&wc[(wn * 128 + b * 32 + arow) * LDT + (ks + 1) * 16 + akq]);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int a = 0; a < 4; ++a)
-#pragma unroll
-        for (int b = 0; b < 4; ++b)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[c][b], af[c][a], acc[a][b], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int i = 2 * ks; i < 2 * ks + 2; ++i) {
-        st16(&xn[(srow0 + i * 32) * LDT + scol], xr[i]);
-        st16(&wn_[(srow0 + i * 32) * LDT + scol], wr[i]);
-      }
-#pragma unroll
-      for (int i = 2 * ks; i < 2 * ks + 2; ++i) {
-        xr[i] = fetch(xres, xoff[i], k2 + scol);
-        wr[i] = fetch(wres, woff[i], k2 + scol);
+      for (int j = 0; j < 16; ++j) {
+        const int a4 = j >> 2, b4 = j & 3;
+        acc[a4][b4] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[c][b4], af[c][a4], acc[a4][b4], 0, 0, 0);
+        const int rd = last ? j - 8 : j;       // slot of the eight fragment reads
+        const int wr_ = last ? j : j - 8;      // slot of the four LDS writes
+        const int ft = last ? j - 4 : j - 12;  // slot of the four global loads
+        if (rd >= 0 && rd < 8) {
+          const u16* xf = last ? xn : xc;
+          const u16* wf = last ? wn_ : wc;
+          const int kk = last ? 0 : (ks + 1) * 16;
+          if (rd < 4) af[nx][rd] = *reinterpret_cast<const bf16x8_t*>(&xf[(wm * 128 + rd * 32 + arow) * LDT + kk + akq]);
+          else bfr[nx][rd - 4] = *reinterpret_cast<const bf16x8_t*>(&wf[(wn * 128 + (rd - 4) * 32 + arow) * LDT + kk + akq]);
+        } else if (wr_ >= 0 && wr_ < 4) {
+          const int i = 2 * ks + (wr_ >> 1);
+          if ((wr_ & 1) == 0) st16(&xn[(srow0 + i * 32) * LDT + scol], xr[i]);
+          else st16(&wn_[(srow0 + i * 32) * LDT + scol], wr[i]);
+        } else if (ft >= 0 && ft < 4) {
+          const int i = 2 * ks + (ft >> 1);
+          if ((ft & 1) == 0) xr[i] = fetch(xres, xoff[i], k2 + scol);
+          else wr[i] = fetch(wres, woff[i], k2 + scol);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (last && j == 3) {
+          asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // LDS only: the global loads stay in flight
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
     }
-    __syncthreads();
   }
 
   // The products were formed as W-tile x X-tile^T, so accumulator element v of a 32 x 32 tile is
   // output column n = (v / 4) * 8 + (lane / 32) * 4 + v % 4 of output row m = lane % 32: a lane holds
   // four consecutive n of one row per group of four registers -> one 8-byte store.
   const bool vec_ok = (ldy & 3) == 0;
+  if (pair_off) {
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const int m = m0 + wm * 128 + a * 32 + (lane & 31);
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int n = n0 + wn * 64 + b * 32 + g * 8 + (lane >> 5) * 4;
+          if (m < M) {
+            float o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = swiglu_bf(round_bf(acc[a][b][4 * g + e]), round_bf(acc[a][b + 2][4 * g + e]));
+            if (vec_ok && n + 3 < N) {
+              uint2 pk;
+              pk.x = pack_bf2(o[0], o[1]);
+              pk.y = pack_bf2(o[2], o[3]);
+              *reinterpret_cast<uint2*>(y + (int64_t)m * ldy + n) = pk;
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                if (n + e < N) y[(int64_t)m * ldy + n + e] = f_to_bf(o[e]);
+            }
+          }
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int a = 0; a < 4; ++a) {
     const int m = m0 + wm * 128 + a * 32 + (lane & 31);
@@ -291,8 +336,9 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
   }
 }
 
+// pair_off != 0: N counts [up; gate] row pairs (see the kernel)
 static int launch_gemm_big(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
-                           hipStream_t s) {
+                           int pair_off, hipStream_t s) {
   constexpr size_t lds = (size_t)2 * (GM + GN) * LDT * sizeof(u16);
   static bool attr_set = false;
   if (!attr_set) {
@@ -301,9 +347,10 @@ static int launch_gemm_big(const void* x, int64_t ldx, const void* w, void* y, i
       return LR_E_LAUNCH;
     attr_set = true;
   }
-  const int tm = (M + GM - 1) / GM, tn = (N + GN - 1) / GN;
+  const int gn = pair_off ? GN / 2 : GN;
+  const int tm = (M + GM - 1) / GM, tn = (N + gn - 1) / gn;
   k_gemm_big<<<dim3((unsigned)(tm * tn)), dim3(256), lds, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy, M, N, K,
-                                                              tm, tn);
+                                                              tm, tn, pair_off);
   return lr_launch_status();
 }
 
@@ -327,7 +374,7 @@ extern "C" int lr_linear_tuned(const void* x, int64_t ldx, const void* w, void* 
   }
   if (!act_swiglu && M >= 512 && N >= 256 && ((M + GM - 1) / GM) * ((N + GN - 1) / GN) >= 192 &&
       (int64_t)GM * ldx * 2 < 0x7fffffff && (int64_t)GN * K * 2 < 0x7fffffff)
-    return launch_gemm_big(x, ldx, w, y, ldy, M, N, K, s);
+    return launch_gemm_big(x, ldx, w, y, ldy, M, N, K, 0, s);
   const dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
   if (grid.y > 65535) return LR_E_UNSUPPORTED;
   if (act_swiglu)
@@ -340,4 +387,32 @@ extern "C" int lr_linear_tuned(const void* x, int64_t ldx, const void* w, void* 
 extern "C" int lr_linear(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
                          int act_swiglu, lr_stream_t stream) {
   return lr_linear_tuned(x, ldx, w, y, ldy, M, N, K, act_swiglu, 0, stream);
+}
+
+// y[M, I] = bf16( bf16(silu(g)) * u ) for [u | g] = x w^T with w = [up; gate] rows (N = 2 I): the MLP's first
+// projection with the activation applied on the way out (utils.py:145-148 without the [M, 2 I] tensor).
+extern "C" int lr_linear_swiglu_out(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
+                                    void* scratch, size_t scratch_bytes, lr_stream_t stream) {
+  LR_REQUIRE_PTR(x);
+  LR_REQUIRE_PTR(w);
+  LR_REQUIRE_PTR(y);
+  if (M <= 0 || N <= 0 || K <= 0 || N % 2 || ldx < K || ldy < N / 2) return LR_E_SHAPE;
+  if (K % 8 || ldx % 8) return LR_E_ALIGN;
+  const int I = N / 2;
+  if (M <= 64) {
+    lr_projection_t pr;
+    pr.x = x; pr.ldx = ldx; pr.w = w; pr.y = y; pr.ldy = ldy; pr.N = N; pr.K = K; pr.epilogue = LR_EPI_SWIGLU; pr.rope = nullptr;
+    const int rc = lr_linear_multi(&pr, 1, M, stream);
+    if (rc != LR_E_UNSUPPORTED) return rc;
+  }
+  if (M >= 512 && I >= 128 && ((M + GM - 1) / GM) * ((I + GN / 2 - 1) / (GN / 2)) >= 192 &&
+      (int64_t)GM * ldx * 2 < 0x7fffffff && ((int64_t)I + GN) * K * 2 < 0x7fffffff)
+    return launch_gemm_big(x, ldx, w, y, ldy, M, I, K, I, (hipStream_t)stream);
+  // other sizes: the projection into `scratch` [M, N], then the activation
+  LR_REQUIRE_PTR(scratch);
+  if (scratch_bytes < (size_t)M * N * sizeof(u16)) return LR_E_SHAPE;
+  if (ldy != I) return LR_E_UNSUPPORTED;  // lr_swiglu writes dense rows
+  const int rc = lr_linear(x, ldx, w, scratch, N, M, N, K, 0, stream);
+  if (rc != LR_OK) return rc;
+  return lr_swiglu(scratch, N, y, M, I, stream);
 }

@@ -26,6 +26,8 @@ _PROTOS = {
     "lr_linear_tuned": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int,
                                 c_void_p]),
     "lr_linear_multi": (c_int, [c_void_p, c_int, c_int, c_void_p]),
+    "lr_linear_swiglu_out": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p,
+                                     c_size_t, c_void_p]),
     "lr_linear_fp8_scratch_bytes": (c_size_t, [c_int, c_int, c_int]),
     "lr_linear_fp8": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p,
                               c_size_t, c_void_p]),
@@ -264,6 +266,19 @@ def linear_swiglu(h: torch.Tensor, w: torch.Tensor, out: torch.Tensor, act: torc
         act = h.new_empty(M, two_k // 2)
     swiglu(h, act)
     return linear(act, w, out)
+
+
+def linear_swiglu_out(x: torch.Tensor, w1: torch.Tensor, act: torch.Tensor, scratch: torch.Tensor = None):
+    """act[M, I] = silu(g) * u for [u | g] = x @ w1^T, w1 = [up; gate] rows: the activation is applied in the
+    projection's epilogue where the shape allows (lr_linear_swiglu_out); `scratch` [M, 2 I] serves the rest."""
+    M, K, ldx = _rows_ld(x)
+    N, Kw = w1.shape
+    Mo, Io, ldy = _rows_ld(act)
+    assert w1.is_contiguous() and Kw == K and N % 2 == 0 and (Mo, Io) == (M, N // 2), (x.shape, w1.shape, act.shape)
+    sp, sb = (None, 0) if scratch is None else (_dev(scratch), scratch.numel() * scratch.element_size())
+    _check(load().lr_linear_swiglu_out(_dev(x), ldx, _dev(w1), _dev(act), ldy, M, N, K, sp, sb, _stream()),
+           "lr_linear_swiglu_out")
+    return act
 
 
 def module_linear(x: torch.Tensor, mod, out: torch.Tensor):

@@ -183,7 +183,13 @@ class GPTBase(nn.Module):
 
     def _mlp(self, ws: Workspace, blk, out: Tensor, xn: Optional[Tensor] = None):
         ff = blk.feed_forward
-        _hip.module_linear(ws.xn if xn is None else xn, ff.w1, ws.h)
+        xin = ws.xn if xn is None else xn
+        if xin.shape[0] > 4 and not hasattr(ff.w1, "scales"):
+            # the activation in the first projection's epilogue; up to 4 rows it is fused into w2's GEMV instead
+            _hip.linear_swiglu_out(xin, ff.w1.weight, ws.act, ws.h)
+            _hip.module_linear(ws.act, ff.w2, out)
+            return
+        _hip.module_linear(xin, ff.w1, ws.h)
         _hip.module_linear_swiglu(ws.h, ff.w2, out, ws.act)
 
     # -- greedy decoding helper ---------------------------------------------------------------------

@@ -251,6 +251,28 @@ def test_linear_multi_rope_kv_epilogue_reports_a_position_outside_the_cache(hip)
     assert torch.equal(q, plain) and torch.equal(kc, kc0) and torch.equal(vc, vc0)
 
 
+@pytest.mark.parametrize("M,D,I", [(5, 264, 56), (64, 1024, 520), (100, 520, 136), (512, 4096, 14336 // 4), (700, 328, 1000),
+                                   (2048, 1024, 3584)])
+def test_linear_swiglu_out_equals_projection_then_swiglu(hip, M, D, I):
+    """The first MLP projection with the activation in its epilogue -- the streaming kernel's row pairs (M <= 64), the
+    256 x 256 tile GEMM on tiles of 128 pairs (M >= 512, ragged edges included), the two-step fallback in between --
+    against the oracle's ops, and bit for bit against lr_linear followed by lr_swiglu."""
+    x, w1 = rnd(M, D, seed=50), rnd(2 * I, D, seed=51, scale=0.03)
+    act = torch.full((M, I), 3.0, dtype=BF, device=DEV)
+    scratch = torch.empty(M, 2 * I, dtype=BF, device=DEV)
+    hip.linear_swiglu_out(x, w1, act, scratch)
+    h = torch.empty(M, 2 * I, dtype=BF, device=DEV)
+    hip.linear(x, w1, h)
+    two_step = torch.empty(M, I, dtype=BF, device=DEV)
+    hip.swiglu(h, two_step)
+    want = swiglu_of_projection_ref(x, w1)
+    assert torch.isfinite(act.float()).all()
+    assert (act.float() - want.float()).abs().max().item() <= 2.0 ** -6 * want.float().abs().max().item()
+    assert (ulp_diff(act, want) > 1).float().mean().item() < 0.05
+    # same kernel family on both sides (same summation order) wherever the fused form exists: identical bits
+    assert torch.equal(act, two_step)
+
+
 def test_linear_multi_is_deterministic(hip):
     x, w = rnd(64, 8192, seed=36), rnd(1280, 8192, seed=37, scale=0.02)
     ys = []
