@@ -28,9 +28,9 @@ Prints ONE JSON line.  `value` = decoded tokens per second (whole job = the one 
                threads used (the process's CPU share: OMP_NUM_THREADS when set, else every core),
                `host_cpus` = os.cpu_count().
 Measured in the same run and reported as extra keys (not the headline; --no-extras skips them):
-`batched`     : the same rank shard at batch 8 and 64, the 8B model at batch 16 (prompt 1024) and the 405B
-               rank shard at batch 16 (context 4096) -- per-op kernels, hipGraph replay: ms per step,
-               tok/s, algorithmic GB/s and its fraction of 8 TB/s.
+`batched`     : the same rank shard at batch 8 and 64, the 8B model at batch 1 (one-kernel step) and 16 (prompt
+               1024) and the 405B rank shard at batch 16 (context 4096) -- per-op kernels unless noted,
+               hipGraph replay: ms per step, tok/s, algorithmic GB/s and its fraction of 8 TB/s.
 `fp8`         : the same shard with weight-only e4m3 projections at batch 1 (per-op kernels): ms per
                step and the fraction of 8 TB/s on ITS algorithmic bytes (one byte per weight + scales).
 `prefill`     : Ladder-8B, batch 32 x 2048 prompt tokens, causal prefill with last-position logits:
@@ -125,7 +125,7 @@ def extra_batched(bm, model, prompt, T, batches=(8, 64), K=32, W=5):
 
 
 def extra_model_decode(bm, name, B, T, K=16, W=3):
-    """Another decode configuration of the benchmark set, on a model of its own (random weights, per-op kernels)."""
+    """Another decode configuration of the benchmark set, on a model of its own (random weights)."""
     import torch
 
     model = bm._load_model(name, "cuda", torch.bfloat16, seed=0, verbose=False)
@@ -365,6 +365,7 @@ def main():
         torch.cuda.empty_cache()
         out["prefill"] = extra_prefill(bm)
         # the other decode configurations of the benchmark set: the 8B model at batch 16, the 405B rank shard at batch 16
+        out["batched"].append(extra_model_decode(bm, "gpt_ladder:ladder-8b", 1, 1024, K=32, W=5))   # one-kernel step
         out["batched"].append(extra_model_decode(bm, "gpt_ladder:ladder-8b", 16, 1024))
         out["batched"].append(extra_model_decode(bm, "gpt_ladder:ladder-405b-tp8", 16, 4096))
     else:

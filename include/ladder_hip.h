@@ -260,8 +260,9 @@ typedef struct {
 typedef struct {
   int32_t dim, n_layer, n_head, n_kv_head, head_dim, ffn, out_rows, vocab, smax, block_size;
   float eps;
-  int32_t attention_workgroups; /* 0: chosen by the library; > 0: use at least this many workgroups for
-                                   attention (fewer keys each, at most 16) -- part of the workspace layout */
+  int32_t attention_workgroups; /* 0: chosen by the library; > 0: cut the keys into at least this many ranges
+                                   (at most 16), one attention workgroup per range and group of kv heads --
+                                   part of the workspace layout */
   const void *tok_embeddings, *norm, *output, *freqs_cis; /* [vocab, dim], [dim], [out_rows, dim], table */
   const lr_layer_t* layers_dev;                           /* DEVICE array of n_layer entries            */
 } lr_ladder_model_t;

@@ -11,7 +11,7 @@
 // side.  A "slot" t = layer t is, per workgroup,
 //     R += a(t-1), attention norm (redundantly in every workgroup; the residual stream itself
 //         never leaves the workgroup's LDS); wqkv(t) rows
-//     attention workgroups (about one per 128 keys): R += m(t-1), then attention(t) over their key
+//     attention workgroups (about one per 128 keys, and per kv head where a rank has several): R += m(t-1), then attention(t) over their key
 //         range with K/V held in registers -- scores on the matrix cores (v_mfma_f32_32x32x16_bf16,
 //         one tile per 32 keys), fp32 softmax and P.V -- un-normalised partial results; then each of
 //         them merges all partial results for its share of the output elements and publishes bf16
@@ -105,6 +105,7 @@ struct LayerPtrs {
 
 struct StepParams {
   int D, L, Hkv, I, V, vocab, Smax, block_size, B, NA, nqkv;
+  int NAK, NAH;  // NA = NAK key ranges x NAH groups of kv heads: attention workgroup w takes range w % NAK of group w / NAK
   float eps;
   const u16 *tok_emb, *final_norm, *out_w, *rope;
   const LayerPtrs* layers;
@@ -889,7 +890,7 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
                                                   float* s_m, float* s_l) {
   constexpr int LPK = HD / 8, KPW = 64 / LPK;
   const int tid = opaque_tid(), wave = tid >> 6, lane = tid & 63;
-  const int aw = blockIdx.x, NA = p.NA, Hkv = p.Hkv, Hq = Hkv * G;
+  const int aw = (int)blockIdx.x % p.NAK, NA = p.NAK, Hkv = p.Hkv, Hq = Hkv * G;  // key range, ranges per head
   const int n = k1 - k0;
   const bool owner = pos >= k0 && pos < k1;
   const float scale = rsqrtf((float)HD);
@@ -1067,9 +1068,9 @@ template <int M, int HD>
 __device__ __forceinline__ void attention_merge_slice(const StepParams& p, const Coh& coh, int Hq, unsigned tag,
                                                       float* wbuf, int aw) {
   const int tid = opaque_tid(), wave = tid >> 6, lane = tid & 63;
-  const int NA = p.NA, nbh = p.B * Hq;
+  const int NA = p.NAK, nbh = p.B * Hq;  // partial results per head
   const int npairs = nbh * HD / 2;
-  const int per = (npairs + NA - 1) / NA;
+  const int per = (npairs + p.NA - 1) / p.NA;  // every attention workgroup merges a share of the outputs
   const int p0 = aw * per, p1 = p0 + per < npairs ? p0 + per : npairs;
   if (p0 >= p1) return;
   u32x4_t raw[NA_MAX];
@@ -1170,8 +1171,8 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   const bool att_wg = w < NA;
   // attention key range of this workgroup
   const int nkeys = pos + 1;
-  const int chunk = (nkeys + NA - 1) / NA;
-  const int k0 = w * chunk;
+  const int chunk = (nkeys + p.NAK - 1) / p.NAK;
+  const int k0 = (w % p.NAK) * chunk;
   const int k1 = k0 + chunk < nkeys ? k0 + chunk : nkeys;
 
   const int qdim = Hq * HD;
@@ -1239,8 +1240,9 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
       LayerPtrs lcache;  // only the cache pointers are used
       lcache.k_cache = const_cast<u16*>(ring_ptr(lring, t, LP_K_CACHE));
       lcache.v_cache = const_cast<u16*>(ring_ptr(lring, t, LP_V_CACHE));
+      const int hpg = p.Hkv / p.NAH, kvh0 = (w / p.NAK) * hpg;  // this workgroup's kv heads
       for (int b = 0; b < p.B; ++b)
-        for (int kvh = 0; kvh < p.Hkv; ++kvh) {
+        for (int kvh = kvh0; kvh < kvh0 + hpg; ++kvh) {
           attention_load<HD>(p, lcache, b, kvh, k0, k1, pos, kv);
           attention_compute<M, HD, G>(p, coh, lcache, b, kvh, k0, k1, pos, tag, LR_STAMP_PTR, kv,
                                       reinterpret_cast<u32*>(qs), sc, sc_ld, ored, reinterpret_cast<u32*>(knew), vnew,
@@ -1397,10 +1399,49 @@ static int pick_na(int Smax, int hd, int nwg, int want_na) {
   return na;
 }
 
+// How the attention workgroups are laid out: `nak` key ranges times `nah` groups of kv heads.  With one kv
+// head per rank (a TP shard) that is pick_na key ranges.  With several kv heads a workgroup that walked all of
+// them one after the other would keep the weight-streaming workgroups waiting (8B model: 62 us of attention
+// against 34 us of w1 per layer), so every kv head gets workgroups of its own and the key ranges become as long
+// as the registers allow (at most 256 keys), within a quarter of the grid.
+struct AttSplit {
+  int nak, nah;
+};
+static AttSplit pick_split(const lr_ladder_model_t* md, int nwg) {
+  const int hd = md->head_dim, hkv = md->n_kv_head;
+  AttSplit a;
+  if (hkv == 1) {
+    a.nak = pick_na(md->smax, hd, nwg, md->attention_workgroups);
+    a.nah = 1;
+    return a;
+  }
+  const int cap = att_capacity(hd) < 256 ? att_capacity(hd) : 256;
+  a.nak = (md->smax + cap - 1) / cap;
+  if (md->attention_workgroups > a.nak) a.nak = md->attention_workgroups;
+  if (a.nak > NA_MAX) a.nak = NA_MAX;
+  if (a.nak < 1) a.nak = 1;
+  // kv heads per workgroup: whichever division makes the slower of the two sides fastest.  The model (times in
+  // microseconds, measured on the MI355X): the other workgroups stream w1 at about 30 GB/s each; an attention
+  // workgroup needs 4 to get q, 2.5 + 0.04 per key for each of its kv heads, 3 for its share of the merge.
+  const float keys = (float)((md->smax + a.nak - 1) / a.nak);
+  float best = 3.0e38f;
+  a.nah = 1;
+  for (int nah = 1; nah <= hkv; ++nah) {
+    if (hkv % nah || a.nak * nah > nwg / 2) continue;
+    const float t_att = 7.0f + (float)(hkv / nah) * (2.5f + 0.04f * keys);
+    const float t_w1 = 4.0f * (float)md->ffn * (float)md->dim / (float)(nwg - a.nak * nah) / 30.0e3f;
+    const float t = t_att > t_w1 ? t_att : t_w1;
+    if (t < best) { best = t; a.nah = nah; }
+  }
+  if (a.nak < 1) a.nak = 1;
+  if (a.nak * a.nah >= nwg) a.nak = (nwg - 1) / a.nah > 0 ? (nwg - 1) / a.nah : 1;
+  return a;
+}
+
 static Layout make_layout(const lr_ladder_model_t* md, int B, int nwg) {
   const int D = md->dim, Hq = md->n_head, hd = md->head_dim;
   const int nqkv = (Hq + 2 * md->n_kv_head) * hd;
-  const int na = pick_na(md->smax, hd, nwg, md->attention_workgroups);
+  const int na = pick_split(md, nwg).nak;  // partial results per head
   auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
   Layout l;
   size_t o = 0;
@@ -1464,8 +1505,10 @@ static int validate(const lr_ladder_model_t* md, int B) {
   const int nwg = num_cus();
   if (nwg < 2) return LR_E_LAUNCH;
   if (md->dim > NJMAX * nwg) return LR_E_UNSUPPORTED;  // a workgroup's rows of wo / w2 fit one reduction round
-  const int na = pick_na(md->smax, md->head_dim, nwg, md->attention_workgroups);
-  if (na > NA_MAX || (md->smax + na - 1) / na > att_capacity(md->head_dim)) return LR_E_UNSUPPORTED;
+  const AttSplit as = pick_split(md, nwg);
+  if (as.nak > NA_MAX || (md->smax + as.nak - 1) / as.nak > att_capacity(md->head_dim) || as.nak * as.nah >= nwg ||
+      md->n_kv_head % as.nah)
+    return LR_E_UNSUPPORTED;
   if (!md->tok_embeddings || !md->norm || !md->output || !md->freqs_cis || !md->layers_dev) return LR_E_NULL;
   return LR_OK;
 }
@@ -1540,7 +1583,8 @@ extern "C" int lr_ladder_decode_step(const lr_ladder_model_t* md, int batch, con
   StepParams sp;
   sp.D = md->dim; sp.L = md->n_layer; sp.Hkv = md->n_kv_head; sp.I = md->ffn; sp.V = md->out_rows;
   sp.vocab = md->vocab; sp.Smax = md->smax; sp.block_size = md->block_size; sp.B = batch;
-  sp.NA = pick_na(md->smax, md->head_dim, nwg, md->attention_workgroups);
+  const AttSplit as = pick_split(md, nwg);
+  sp.NAK = as.nak; sp.NAH = as.nah; sp.NA = as.nak * as.nah;
   sp.nqkv = (md->n_head + 2 * md->n_kv_head) * md->head_dim;
   sp.eps = md->eps;
   sp.tok_emb = (const u16*)md->tok_embeddings; sp.final_norm = (const u16*)md->norm;
