@@ -54,8 +54,13 @@ template <int MT, int UNITS>
 __global__ __launch_bounds__(NWV * 64) void k_stream_gemm(const Proj p0, const Proj p1, const int M) {
   constexpr int MTILES = MT / 16, KS = KC / 32, NLD = UNITS * 4;
   constexpr int NV = UNITS * MTILES * 4;  // accumulator registers per lane
-  __shared__ __attribute__((aligned(16))) u16 lds[NWV][UNITS * 16 * LROW];
-  static_assert(sizeof(float) * NV * 64 <= sizeof(u16) * UNITS * 16 * LROW, "the partial sums reuse the wave's LDS piece");
+  // From 32 input rows on the inputs too are loaded in whole lines (4 rows x 256 bytes per instruction) and take
+  // the trip through LDS into B-fragment layout: L2 serves whole-line reads 1.5 times as fast as the 16 rows x
+  // 64 bytes a fragment-layout load touches, and at 64 rows the input bytes are twice the weight bytes.
+  constexpr bool XLDS = MT >= 32;
+  constexpr int WPIECE = UNITS * 16 * LROW, XPIECE = XLDS ? MT * LROW : 0;  // elements per wave
+  extern __shared__ __attribute__((aligned(16))) u16 sg_smem[];              // [NWV][WPIECE + XPIECE]
+  static_assert(sizeof(float) * NV * 64 <= sizeof(u16) * WPIECE, "the partial sums reuse the wave's weight piece");
 
   const bool second = (int)blockIdx.x >= p0.nwg;
   const u16* const xg = second ? p1.x : p0.x;
@@ -87,13 +92,24 @@ __global__ __launch_bounds__(NWV * 64) void k_stream_gemm(const Proj p0, const P
     if (pair_off && r >= 16) { rr = r - 16; extra = pair_off; }
     woff[i] = rr < nrows ? (int)(((int64_t)(extra + rr) * K + l16 * 8) * 2) : OOB;
   }
-  int xoff[MTILES];
+  // fragment layout: tile mt, k-step ks <- input row 16 mt + lane % 16, elements 32 ks + 8 (lane / 16) ..;
+  // whole-line layout: instruction i <- input rows 4 i + lane / 16, elements 8 (lane % 16) ..
+  int xoff[XLDS ? MT / 4 : MTILES];
+  if (XLDS) {
 #pragma unroll
-  for (int mt = 0; mt < MTILES; ++mt) {
-    const int m = mt * 16 + l16;
-    xoff[mt] = m < M ? (int)((m * ldx + l4 * 8) * 2) : OOB;
+    for (int i = 0; i < MT / 4; ++i) {
+      const int m = 4 * i + l4;
+      xoff[i] = m < M ? (int)((m * ldx + l16 * 8) * 2) : OOB;
+    }
+  } else {
+#pragma unroll
+    for (int mt = 0; mt < MTILES; ++mt) {
+      const int m = mt * 16 + l16;
+      xoff[mt] = m < M ? (int)((m * ldx + l4 * 8) * 2) : OOB;
+    }
   }
-  u16* const my = lds[wave];
+  u16* const my = sg_smem + wave * (WPIECE + XPIECE);
+  u16* const myx = my + WPIECE;
 
   u32x4_t wr[SETS][NLD];
   u32x4_t xr[2][MTILES][KS];
@@ -114,6 +130,14 @@ __global__ __launch_bounds__(NWV * 64) void k_stream_gemm(const Proj p0, const P
   };
   auto issue_x = [&](int ci, u32x4_t (&dst)[MTILES][KS]) {
     const int k0 = (ci * NWV + wave) * KC;
+    if (XLDS) {
+      const bool kok = k0 + l16 * 8 < K;
+#pragma unroll
+      for (int i = 0; i < MT / 4; ++i)
+        dst[i / KS][i % KS] =
+            __builtin_amdgcn_raw_buffer_load_b128(xres, (kok && xoff[i] != OOB) ? xoff[i] : OOB, k0 * 2, 0);
+      return;
+    }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const bool kok = k0 + ks * 32 + l4 * 8 < K;
@@ -148,23 +172,32 @@ __global__ __launch_bounds__(NWV * 64) void k_stream_gemm(const Proj p0, const P
           af[u][ks] = *reinterpret_cast<const bf16x8_t*>(my + (16 * u + l16) * LROW + ks * 32 + l4 * 8);
       asm volatile("" ::: "memory");
       issue_w(ci + SETS, wr[s]);
+      if (XLDS) {
+#pragma unroll
+        for (int i = 0; i < MT / 4; ++i)
+          *reinterpret_cast<u32x4_t*>(myx + (4 * i + l4) * LROW + l16 * 8) = xr[s & 1][i / KS][i % KS];
+        asm volatile("" ::: "memory");
+      }
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
         for (int mt = 0; mt < MTILES; ++mt) {
-          const bf16x8_t bx = __builtin_bit_cast(bf16x8_t, xr[s & 1][mt][ks]);
+          bf16x8_t bx;
+          if (XLDS) bx = *reinterpret_cast<const bf16x8_t*>(myx + (16 * mt + l16) * LROW + ks * 32 + l4 * 8);
+          else bx = __builtin_bit_cast(bf16x8_t, xr[s & 1][mt][ks]);
 #pragma unroll
           for (int u = 0; u < UNITS; ++u)
             acc[u][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[u][ks], bx, acc[u][mt], 0, 0, 0);
         }
+      if (XLDS) asm volatile("" ::: "memory");
     }
   }
 
   // ---- the waves' partial sums meet in LDS (accumulator element e of tile (u, mt): band row
   //      16 u + 4 (lane / 16) + e, input row 16 mt + lane % 16) and are added in wave order
   __syncthreads();
-  float* const red = reinterpret_cast<float*>(&lds[0][0]);
-  constexpr int WSTRIDE = UNITS * 16 * LROW / 2;  // floats per wave piece
+  float* const red = reinterpret_cast<float*>(sg_smem);
+  constexpr int WSTRIDE = (WPIECE + XPIECE) / 2;  // floats per wave piece
 #pragma unroll
   for (int u = 0; u < UNITS; ++u)
 #pragma unroll
@@ -260,11 +293,23 @@ static void plan(Proj& p, int M, int cap, int ncu) {
   p.nwg = (items + rpw - 1) / rpw;
 }
 
+template <int MT, int UNITS>
+static int launch_units(Proj& a, Proj& b, int M, hipStream_t s) {
+  const size_t lds = (size_t)NWV * (UNITS * 16 * LROW + (MT >= 32 ? MT * LROW : 0)) * sizeof(u16);
+  static bool attr_set = false;
+  if (!attr_set && lds > 64 * 1024) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_stream_gemm<MT, UNITS>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return LR_E_LAUNCH;
+    attr_set = true;
+  }
+  k_stream_gemm<MT, UNITS><<<dim3((unsigned)(a.nwg + b.nwg)), dim3(NWV * 64), lds, s>>>(a, b, M);
+  return LR_OK;
+}
+
 template <int MT>
-static void launch(Proj& a, Proj& b, int M, int units, hipStream_t s) {
-  const dim3 grid((unsigned)(a.nwg + b.nwg));
-  if (units == 2) k_stream_gemm<MT, 2><<<grid, dim3(NWV * 64), 0, s>>>(a, b, M);
-  else k_stream_gemm<MT, 1><<<grid, dim3(NWV * 64), 0, s>>>(a, b, M);
+static int launch(Proj& a, Proj& b, int M, int units, hipStream_t s) {
+  return units == 2 ? launch_units<MT, 2>(a, b, M, s) : launch_units<MT, 1>(a, b, M, s);
 }
 
 }  // namespace
@@ -318,8 +363,7 @@ extern "C" int lr_linear_multi(const lr_projection_t* proj, int n_proj, int M, l
   const int units = (any_pair || !all_thin) ? 2 : 1;
   for (int i = 0; i < n_proj; ++i) plan(pr[i], M, pr[i].pair_off ? 16 : 16 * units, ncu);
   hipStream_t s = (hipStream_t)stream;
-  if (M <= 16) launch<16>(pr[0], pr[1], M, units, s);
-  else if (M <= 32) launch<32>(pr[0], pr[1], M, units, s);
-  else launch<64>(pr[0], pr[1], M, units, s);
-  return lr_launch_status();
+  const int rc = M <= 16 ? launch<16>(pr[0], pr[1], M, units, s)
+                 : (M <= 32 ? launch<32>(pr[0], pr[1], M, units, s) : launch<64>(pr[0], pr[1], M, units, s));
+  return rc != LR_OK ? rc : lr_launch_status();
 }
