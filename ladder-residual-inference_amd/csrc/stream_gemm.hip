@@ -29,6 +29,9 @@ constexpr int NWV = 4;         // waves per workgroup
 constexpr int SETS = 4;        // weight chunks in flight per wave
 constexpr int LROW = KC + 8;   // LDS row length in elements (272 bytes)
 constexpr int OOB = (int)0x80000000;  // a buffer offset beyond every resource: the load returns zero, untouched memory
+#ifndef LR_SG_XLDS_MIN
+#define LR_SG_XLDS_MIN 32
+#endif
 #ifndef LR_SG_W_AUX
 #define LR_SG_W_AUX 2          // weights: non-temporal (every line is used exactly once)
 #endif
@@ -57,7 +60,7 @@ __global__ __launch_bounds__(NWV * 64) void k_stream_gemm(const Proj p0, const P
   // From 32 input rows on the inputs too are loaded in whole lines (4 rows x 256 bytes per instruction) and take
   // the trip through LDS into B-fragment layout: L2 serves whole-line reads 1.5 times as fast as the 16 rows x
   // 64 bytes a fragment-layout load touches, and at 64 rows the input bytes are twice the weight bytes.
-  constexpr bool XLDS = MT >= 32;
+  constexpr bool XLDS = MT >= LR_SG_XLDS_MIN;
   constexpr int WPIECE = UNITS * 16 * LROW, XPIECE = XLDS ? MT * LROW : 0;  // elements per wave
   extern __shared__ __attribute__((aligned(16))) u16 sg_smem[];              // [NWV][WPIECE + XPIECE]
   static_assert(sizeof(float) * NV * 64 <= sizeof(u16) * WPIECE, "the partial sums reuse the wave's weight piece");
@@ -295,7 +298,7 @@ static void plan(Proj& p, int M, int cap, int ncu) {
 
 template <int MT, int UNITS>
 static int launch_units(Proj& a, Proj& b, int M, hipStream_t s) {
-  const size_t lds = (size_t)NWV * (UNITS * 16 * LROW + (MT >= 32 ? MT * LROW : 0)) * sizeof(u16);
+  const size_t lds = (size_t)NWV * (UNITS * 16 * LROW + (MT >= LR_SG_XLDS_MIN ? MT * LROW : 0)) * sizeof(u16);
   static bool attr_set = false;
   if (!attr_set && lds > 64 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_stream_gemm<MT, UNITS>),
