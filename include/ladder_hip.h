@@ -152,6 +152,18 @@ int lr_linear_multi(const lr_projection_t* projections, int n_projections, int M
 int lr_linear_swiglu_out(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
                          void* scratch, size_t scratch_bytes, lr_stream_t stream);
 
+/* lr_attn_decode and one projection of lr_linear_multi in ONE launch: the first workgroups of the grid are the
+ * attention's (split, kv head, sequence) items, the rest the bands of the projection, so the projection's weight
+ * stream fills the chip while the attention waits for the KV cache.  For a ladder block, whose up/gate
+ * projection does not depend on the block's own attention (gpt_ladder_TP.py:339-349: the reference overlaps
+ * the attention's all-reduce with the MLP for the same reason); the two halves must be independent of each
+ * other.  Same bits as lr_attn_decode(q, ..., y) followed by lr_linear_multi(projection, 1, M).
+ * Arguments as there.  LR_E_UNSUPPORTED (nothing launched): M > 16, an LR_EPI_ROPE_KV projection (it would write
+ * the cache the attention reads), more than 8 q heads per kv head -- the caller then makes the two calls. */
+int lr_attn_decode_beside(const void* q, int64_t ldq, const void* k_cache, const void* v_cache, const int32_t* pos,
+                          void* y, int64_t ldy, int B, int Hq, int Hkv, int hd, int Smax, void* scratch,
+                          size_t scratch_bytes, const lr_projection_t* projection, int M, lr_stream_t stream);
+
 /* Weight-only fp8 linear:  y[m, n] = bf16( bf16( sum_k x[m, k] * w8[n, k] ) * scales[n] ).
  * w8 [N, K] dense float8 e4m3 (OCP "e4m3fn": bias 7, no infinities, max 448), one byte per weight;
  * scales [N] bf16, one per output row; x, y bf16 as in lr_linear.  K % 16 == 0.

@@ -16,7 +16,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "gpt_fast", "libladder_hip.so")
 PROF_LIB = os.path.join(HERE, "gpt_fast", "libladder_hip_prof.so")
-HEADERS = [os.path.join(CSRC, h) for h in ("lr_common.h", "attn_decode_item.h")] + \
+HEADERS = [os.path.join(CSRC, h) for h in ("lr_common.h", "attn_decode_item.h", "stream_band.h")] + \
     [os.path.join(HERE, "..", "include", "ladder_hip.h")]
 
 FLAGS = [
@@ -69,8 +69,8 @@ def build_step_profile(force=False, verbose=True):
     workgroup and phase (-DLR_STEP_PROFILE; read by step_phases.py).  The product library carries none of it."""
     build(force=force, verbose=False)
     obj, changed = _compile(os.path.join(CSRC, "ladder_step.hip"), force, ("-DLR_STEP_PROFILE",), "_prof")
-    objs = [os.path.join(OBJ, f) for f in sorted(os.listdir(OBJ))
-            if f.endswith(".o") and f not in ("ladder_step.o", "ladder_step_prof.o")] + [obj]
+    objs = [os.path.join(OBJ, f.replace(".hip", ".o")) for f in sorted(os.listdir(CSRC))
+            if f.endswith(".hip") and f != "ladder_step.hip"] + [obj]
     if force or changed or _stale(PROF_LIB, objs):
         r = subprocess.run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PROF_LIB] + objs,
                            capture_output=True, text=True)

@@ -1,0 +1,320 @@
+// The band of the weight-streaming matrix-core kernel as a device function, and what its callers share on the host
+// (stream_gemm.hip launches bands only; decode_pair.hip runs decode-attention items beside them).
+#pragma once
+#include "lr_common.h"
+
+namespace {
+
+
+constexpr int KC = 128;        // k elements per chunk
+constexpr int NWV = 4;         // waves per workgroup
+constexpr int SETS = 4;        // weight chunks in flight per wave
+constexpr int LROW = KC + 8;   // LDS row length in elements (272 bytes)
+constexpr int OOB = (int)0x80000000;  // a buffer offset beyond every resource: the load returns zero, untouched memory
+#ifndef LR_SG_XLDS_MIN
+#define LR_SG_XLDS_MIN 32
+#endif
+#ifndef LR_SG_W_AUX
+#define LR_SG_W_AUX 2          // weights: non-temporal (every line is used exactly once)
+#endif
+
+struct Proj {
+  const u16* x;
+  const u16* w;
+  u16* y;
+  int64_t ldx, ldy;
+  int N, K;      // weight rows, row length
+  int rpw;       // rows (row pairs if pair_off) per workgroup
+  int pair_off;  // 0, or the distance from an up row to its gate row (= outputs)
+  int nwg;       // workgroups of this projection
+  // RoPE + KV-cache epilogue of a fused q/k/v projection (rope_table == nullptr: none)
+  const u16* rope_table;
+  const int32_t* pos;
+  u16 *k_cache, *v_cache;
+  int32_t* err;
+  int Hq, Hkv, hd, Smax, block_size;
+};
+
+template <int MT, int UNITS>
+constexpr size_t stream_band_lds_bytes() {
+  return (size_t)NWV * (UNITS * 16 * LROW + (MT >= LR_SG_XLDS_MIN ? MT * LROW : 0)) * sizeof(u16);
+}
+
+// One band of one projection, by the 256 lanes of a workgroup.  `sg_smem`: stream_band_lds_bytes<MT, UNITS>() bytes of LDS.
+template <int MT, int UNITS>
+__device__ __forceinline__ void stream_band(const Proj& p, const int M, const int band, u16* sg_smem) {
+  constexpr int MTILES = MT / 16, KS = KC / 32, NLD = UNITS * 4;
+  constexpr int NV = UNITS * MTILES * 4;  // accumulator registers per lane
+  // From 32 input rows on the inputs too are loaded in whole lines (4 rows x 256 bytes per instruction) and take
+  // the trip through LDS into B-fragment layout: L2 serves whole-line reads 1.5 times as fast as the 16 rows x
+  // 64 bytes a fragment-layout load touches, and at 64 rows the input bytes are twice the weight bytes.
+  constexpr bool XLDS = MT >= LR_SG_XLDS_MIN;
+  constexpr int WPIECE = UNITS * 16 * LROW, XPIECE = XLDS ? MT * LROW : 0;  // elements per wave
+  // sg_smem: [NWV][WPIECE + XPIECE]
+  static_assert(sizeof(float) * NV * 64 <= sizeof(u16) * WPIECE, "the partial sums reuse the wave's weight piece");
+
+  const u16* const xg = p.x;
+  const u16* const wg_ = p.w;
+  u16* const yg = p.y;
+  const int64_t ldx = p.ldx, ldy = p.ldy;
+  const int N = p.N, K = p.K, rpw = p.rpw;
+  const int pair_off = p.pair_off;
+  const u16* const rope_table = p.rope_table;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l16 = lane & 15, l4 = lane >> 4;
+  const int n_out = pair_off ? pair_off : N;         // output columns
+  const int n0 = band * rpw;                          // first row (pair) of the band
+  const int nrows = n_out - n0 < rpw ? n_out - n0 : rpw;
+
+  // ---- lane constants of the weight loads: instruction i covers band rows 4 i .. 4 i + 3 (in pair mode
+  //      unit 0 holds the up rows, unit 1 the gate rows of the same pairs)
+  const __amdgpu_buffer_rsrc_t wres =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<u16*>(wg_ + (int64_t)n0 * K), 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc(const_cast<u16*>(xg), 0, 0x7fffffff, 0x00020000);
+  int woff[NLD];
+#pragma unroll
+  for (int i = 0; i < NLD; ++i) {
+    const int r = 4 * i + l4;  // row inside the LDS piece
+    int rr = r, extra = 0;
+    if (pair_off && r >= 16) { rr = r - 16; extra = pair_off; }
+    woff[i] = rr < nrows ? (int)(((int64_t)(extra + rr) * K + l16 * 8) * 2) : OOB;
+  }
+  // fragment layout: tile mt, k-step ks <- input row 16 mt + lane % 16, elements 32 ks + 8 (lane / 16) ..;
+  // whole-line layout: instruction i <- input rows 4 i + lane / 16, elements 8 (lane % 16) ..
+  int xoff[XLDS ? MT / 4 : MTILES];
+  if (XLDS) {
+#pragma unroll
+    for (int i = 0; i < MT / 4; ++i) {
+      const int m = 4 * i + l4;
+      xoff[i] = m < M ? (int)((m * ldx + l16 * 8) * 2) : OOB;
+    }
+  } else {
+#pragma unroll
+    for (int mt = 0; mt < MTILES; ++mt) {
+      const int m = mt * 16 + l16;
+      xoff[mt] = m < M ? (int)((m * ldx + l4 * 8) * 2) : OOB;
+    }
+  }
+  u16* const my = sg_smem + wave * (WPIECE + XPIECE);
+  u16* const myx = my + WPIECE;
+
+  u32x4_t wr[SETS][NLD];
+  u32x4_t xr[2][MTILES][KS];
+  f32x4_t acc[UNITS][MTILES];
+#pragma unroll
+  for (int u = 0; u < UNITS; ++u)
+#pragma unroll
+    for (int mt = 0; mt < MTILES; ++mt) acc[u][mt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+  // chunk ci of this wave starts at k0 = (ci * NWV + wave) * KC; what lies beyond K reads as zero (no
+  // branch around a load: the number of loads in flight is fixed, so the waits between chunks are exact)
+  auto issue_w = [&](int ci, u32x4_t (&dst)[NLD]) {
+    const int k0 = (ci * NWV + wave) * KC;
+    const bool kok = k0 + l16 * 8 < K;
+#pragma unroll
+    for (int i = 0; i < NLD; ++i)
+      dst[i] = __builtin_amdgcn_raw_buffer_load_b128(wres, (kok && woff[i] != OOB) ? woff[i] : OOB, k0 * 2, LR_SG_W_AUX);
+  };
+  auto issue_x = [&](int ci, u32x4_t (&dst)[MTILES][KS]) {
+    const int k0 = (ci * NWV + wave) * KC;
+    if (XLDS) {
+      const bool kok = k0 + l16 * 8 < K;
+#pragma unroll
+      for (int i = 0; i < MT / 4; ++i)
+        dst[i / KS][i % KS] =
+            __builtin_amdgcn_raw_buffer_load_b128(xres, (kok && xoff[i] != OOB) ? xoff[i] : OOB, k0 * 2, 0);
+      return;
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const bool kok = k0 + ks * 32 + l4 * 8 < K;
+#pragma unroll
+      for (int mt = 0; mt < MTILES; ++mt)
+        dst[mt][ks] = __builtin_amdgcn_raw_buffer_load_b128(xres, (kok && xoff[mt] != OOB) ? xoff[mt] : OOB,
+                                                           (k0 + ks * 32) * 2, 0);
+    }
+  };
+
+  const int nck = (K + KC - 1) / KC;
+  const int nch = wave < nck ? (nck - wave + NWV - 1) / NWV : 0;  // chunks of this wave
+  issue_x(0, xr[0]);
+#pragma unroll
+  for (int s = 0; s < SETS; ++s) issue_w(s, wr[s]);
+  for (int c0 = 0; c0 < nch; c0 += SETS) {
+#pragma unroll
+    for (int s = 0; s < SETS; ++s) {
+      const int ci = c0 + s;
+      issue_x(ci + 1, xr[(s + 1) & 1]);
+      // ---- this chunk's weights: registers -> LDS (row-major) -> A fragments
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int i = 0; i < NLD; ++i)
+        *reinterpret_cast<u32x4_t*>(my + (4 * i + l4) * LROW + l16 * 8) = wr[s][i];
+      asm volatile("" ::: "memory");
+      bf16x8_t af[UNITS][KS];
+#pragma unroll
+      for (int u = 0; u < UNITS; ++u)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          af[u][ks] = *reinterpret_cast<const bf16x8_t*>(my + (16 * u + l16) * LROW + ks * 32 + l4 * 8);
+      asm volatile("" ::: "memory");
+      issue_w(ci + SETS, wr[s]);
+      if (XLDS) {
+#pragma unroll
+        for (int i = 0; i < MT / 4; ++i)
+          *reinterpret_cast<u32x4_t*>(myx + (4 * i + l4) * LROW + l16 * 8) = xr[s & 1][i / KS][i % KS];
+        asm volatile("" ::: "memory");
+      }
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int mt = 0; mt < MTILES; ++mt) {
+          bf16x8_t bx;
+          if (XLDS) bx = *reinterpret_cast<const bf16x8_t*>(myx + (16 * mt + l16) * LROW + ks * 32 + l4 * 8);
+          else bx = __builtin_bit_cast(bf16x8_t, xr[s & 1][mt][ks]);
+#pragma unroll
+          for (int u = 0; u < UNITS; ++u)
+            acc[u][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[u][ks], bx, acc[u][mt], 0, 0, 0);
+        }
+      if (XLDS) asm volatile("" ::: "memory");
+    }
+  }
+
+  // ---- the waves' partial sums meet in LDS (accumulator element e of tile (u, mt): band row
+  //      16 u + 4 (lane / 16) + e, input row 16 mt + lane % 16) and are added in wave order
+  __syncthreads();
+  float* const red = reinterpret_cast<float*>(sg_smem);
+  constexpr int WSTRIDE = (WPIECE + XPIECE) / 2;  // floats per wave piece
+#pragma unroll
+  for (int u = 0; u < UNITS; ++u)
+#pragma unroll
+    for (int mt = 0; mt < MTILES; ++mt)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) red[wave * WSTRIDE + ((u * MTILES + mt) * 4 + e) * 64 + lane] = acc[u][mt][e];
+  __syncthreads();
+  const int rows_out = pair_off ? 16 : 16 * UNITS;
+  if (rope_table != nullptr) {
+    // The fused q/k/v projection of a decode step (one token per sequence: input row m is sequence m):
+    // what lr_rope_kv_write would do to the stored row, done here on the (even, odd) output pairs.  A
+    // position outside the cache or the table: the plain projection is stored, the error word is set.
+    const Proj& pp = p;
+    const int hd = pp.hd, nq = pp.Hq * hd, nkv = pp.Hkv * hd;
+    const int ps = pp.pos[0];
+    const bool in_range = ps >= 0 && ps < pp.Smax && ps < pp.block_size;
+    if (!in_range && pp.err && band == 0 && tid == 0) *pp.err = LR_DEV_POS_RANGE;
+    for (int o = tid; o < (rows_out / 2) * MT; o += NWV * 64) {
+      const int r = 2 * (o % (rows_out / 2)), m = o / (rows_out / 2);
+      if (r >= nrows || m >= M) continue;
+      const int mt = m >> 4, ln = ((r & 15) >> 2) * 16 + (m & 15), e = r & 3, u = r >> 4;
+      float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+      for (int wv = 0; wv < NWV; ++wv) {
+        s0 += red[wv * WSTRIDE + ((u * MTILES + mt) * 4 + e) * 64 + ln];
+        s1 += red[wv * WSTRIDE + ((u * MTILES + mt) * 4 + e + 1) * 64 + ln];
+      }
+      const float x0 = round_bf(s0), x1 = round_bf(s1);
+      const int n = n0 + r;
+      u32 plain = pack_bf2(x0, x1), out = plain;
+      if (in_range) {
+        const int sect = n < nq ? 0 : (n < nq + nkv ? 1 : 2);
+        const int cc = n - (sect == 0 ? 0 : (sect == 1 ? nq : nq + nkv));
+        const int h = cc / hd, d = cc - h * hd;
+        if (sect < 2) {
+#pragma clang fp contract(off)
+          const u32 cs = *reinterpret_cast<const u32*>(rope_table + (int64_t)ps * hd + d);
+          const float c = bf_lo(cs), sn = bf_hi(cs);
+          const float a = x0 * c, b = x1 * sn, dd = x1 * c, ee = x0 * sn;
+          out = pack_bf2(a - b, dd + ee);
+        }
+        if (sect == 0) plain = out;  // q is rotated in place; k and v stay as projected, the cache gets them
+        if (sect == 1) *reinterpret_cast<u32*>(pp.k_cache + (((int64_t)m * pp.Hkv + h) * pp.Smax + ps) * hd + d) = out;
+        if (sect == 2) *reinterpret_cast<u32*>(pp.v_cache + (((int64_t)m * pp.Hkv + h) * pp.Smax + ps) * hd + d) = plain;
+      }
+      *reinterpret_cast<u32*>(yg + (int64_t)m * ldy + n) = plain;
+    }
+    return;
+  }
+  for (int o = tid; o < rows_out * MT; o += NWV * 64) {
+    const int r = o % rows_out, m = o / rows_out;
+    if (r >= nrows || m >= M) continue;
+    const int mt = m >> 4, ln = ((r & 15) >> 2) * 16 + (m & 15), e = r & 3, u = r >> 4;
+    float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+    for (int wv = 0; wv < NWV; ++wv) s0 += red[wv * WSTRIDE + ((u * MTILES + mt) * 4 + e) * 64 + ln];
+    if (pair_off) {
+      if (UNITS == 2) {
+#pragma unroll
+        for (int wv = 0; wv < NWV; ++wv) s1 += red[wv * WSTRIDE + ((MTILES + mt) * 4 + e) * 64 + ln];
+      }
+      yg[(int64_t)m * ldy + n0 + r] = f_to_bf(swiglu_bf(round_bf(s0), round_bf(s1)));
+    } else {
+      yg[(int64_t)m * ldy + n0 + r] = f_to_bf(s0);
+    }
+  }
+}
+
+static int sb_num_cus() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0;
+    n = prop.multiProcessorCount;
+  }
+  return n;
+}
+
+// Rows per workgroup: the rows are spread evenly over whole rounds of the CUs, at most `cap` per
+// workgroup; with few weight rows and many input rows a band is not made thinner than `floor_rows`
+// (every band re-reads all input rows from L2).
+static void plan(Proj& p, int M, int cap, int ncu) {
+  // (the RoPE epilogue works on output pairs: bands of an even number of rows)
+  const int items = p.pair_off ? p.pair_off : p.N;
+  const int rounds = (items + ncu * cap - 1) / (ncu * cap);
+  int rpw = (items + ncu * rounds - 1) / (ncu * rounds);
+  const int floor_rows = M > 32 ? 16 : (M > 16 ? 8 : 4);
+  if (rpw < floor_rows) rpw = floor_rows;
+  if (p.rope_table) rpw = (rpw + 1) & ~1;
+  if (rpw > cap) rpw = cap;
+  p.rpw = rpw;
+  p.nwg = (items + rpw - 1) / rpw;
+}
+
+// lr_projection_t -> Proj (validated; rpw / nwg are set by plan())
+static int sb_fill_projection(const lr_projection_t& q, Proj& p) {
+  LR_REQUIRE_PTR(q.x);
+  LR_REQUIRE_PTR(q.w);
+  LR_REQUIRE_PTR(q.y);
+  if (q.N <= 0 || q.K <= 0 || q.ldx < q.K) return LR_E_SHAPE;
+  if (q.epilogue != LR_EPI_NONE && q.epilogue != LR_EPI_SWIGLU && q.epilogue != LR_EPI_ROPE_KV) return LR_E_SHAPE;
+  const bool pair = q.epilogue == LR_EPI_SWIGLU;
+  if (pair && q.N % 2) return LR_E_SHAPE;
+  if (q.ldy < (pair ? q.N / 2 : q.N)) return LR_E_SHAPE;
+  if (q.K % 8 || q.ldx % 8) return LR_E_ALIGN;
+  // offsets inside a band and inside the input rows are 32-bit
+  if ((int64_t)64 * q.ldx * 2 >= 0x7fffffff || ((int64_t)(pair ? q.N / 2 : 0) + 64) * q.K * 2 >= 0x7fffffff)
+    return LR_E_UNSUPPORTED;
+  p = Proj{};
+  p.x = (const u16*)q.x; p.w = (const u16*)q.w; p.y = (u16*)q.y;
+  p.ldx = q.ldx; p.ldy = q.ldy; p.N = q.N; p.K = q.K;
+  p.pair_off = pair ? q.N / 2 : 0;
+  if (q.epilogue == LR_EPI_ROPE_KV) {
+    const lr_rope_kv_t* r = q.rope;
+    if (r == nullptr || r->pos == nullptr) return LR_E_NULL;
+    LR_REQUIRE_PTR(r->table);
+    LR_REQUIRE_PTR(r->k_cache);
+    LR_REQUIRE_PTR(r->v_cache);
+    if (r->n_head <= 0 || r->n_kv_head <= 0 || r->head_dim <= 0 || r->smax <= 0 || r->block_size <= 0 ||
+        (int64_t)(r->n_head + 2 * r->n_kv_head) * r->head_dim != q.N || q.ldy % 2)
+      return LR_E_SHAPE;
+    if (r->head_dim % 8) return LR_E_ALIGN;
+    p.rope_table = (const u16*)r->table; p.pos = r->pos; p.k_cache = (u16*)r->k_cache; p.v_cache = (u16*)r->v_cache;
+    p.err = r->err; p.Hq = r->n_head; p.Hkv = r->n_kv_head; p.hd = r->head_dim; p.Smax = r->smax;
+    p.block_size = r->block_size;
+  }
+  return LR_OK;
+}
+
+}  // namespace

@@ -37,6 +37,8 @@ _PROTOS = {
     "lr_attn_decode_scratch_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "lr_attn_decode": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int,
                                c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "lr_attn_decode_beside": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,
+                                      c_int, c_int, c_int, c_void_p, c_size_t, c_void_p, c_int, c_void_p]),
     "lr_attn_decode_static": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,
                                       c_int, c_int, c_int, c_void_p]),
     "lr_attn_prefill": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,
@@ -59,6 +61,9 @@ class LadderModelDesc(ctypes.Structure):
     _fields_ = [(n, c_int32) for n in ("dim", "n_layer", "n_head", "n_kv_head", "head_dim", "ffn", "out_rows", "vocab",
                                        "smax", "block_size")] + [("eps", c_float), ("attention_workgroups", c_int32)] + \
                [(n, c_void_p) for n in ("tok_embeddings", "norm", "output", "freqs_cis", "layers_dev")]
+
+
+E_UNSUPPORTED = -4   # LR_E_UNSUPPORTED of include/ladder_hip.h
 
 
 class LadderHipError(RuntimeError):
@@ -213,6 +218,11 @@ def linear_multi(*projections):
     EPI_SWIGLU -> w holds [up; gate] rows and out [M, N / 2] = silu(gate) * up; or, for the fused q/k/v
     projection of a decode step, (x, w, out, rope_kv_epilogue(...)): q rotated in out, k and v into the cache
     (lr_linear_multi)."""
+    arr, M, _keep = _projection_array(projections)
+    _check(load().lr_linear_multi(ctypes.cast(arr, c_void_p), len(projections), M, _stream()), "lr_linear_multi")
+
+
+def _projection_array(projections):
     arr = (_Projection * len(projections))()
     M = None
     keep = []
@@ -230,7 +240,7 @@ def linear_multi(*projections):
         M = m
         arr[i] = _Projection(_dev(x), ldx, _dev(w), _dev(out), ldy, N, K, epi,
                              ctypes.pointer(rope) if rope is not None else None)
-    _check(load().lr_linear_multi(ctypes.cast(arr, c_void_p), len(projections), M, _stream()), "lr_linear_multi")
+    return arr, M, keep
 
 
 def linear_fp8(x: torch.Tensor, w8: torch.Tensor, scales: torch.Tensor, out: torch.Tensor):
@@ -370,6 +380,23 @@ def attn_decode(q, k_cache, v_cache, pos, y, scratch, B, Hq, Hkv, hd):
     return y
 
 
+def attn_decode_beside(q, k_cache, v_cache, pos, y, scratch, B, Hq, Hkv, hd, projection) -> bool:
+    """attn_decode and linear_multi(projection) in one launch (lr_attn_decode_beside); the two must not depend
+    on each other.  False, with nothing launched, when the library has no such kernel for the shape."""
+    _, _, ldq = _rows_ld(q)
+    _, _, ldy = _rows_ld(y)
+    Smax = k_cache.shape[2]
+    assert pos.dtype == torch.int32 and pos.numel() == 1 and scratch.dtype == torch.float32
+    arr, M, _keep = _projection_array((projection,))
+    rc = load().lr_attn_decode_beside(_dev(q), ldq, _dev(k_cache), _dev(v_cache), pos.data_ptr(), _dev(y), ldy, B, Hq,
+                                      Hkv, hd, Smax, scratch.data_ptr(), scratch.numel() * 4,
+                                      ctypes.cast(arr, c_void_p), M, _stream())
+    if rc == E_UNSUPPORTED:
+        return False
+    _check(rc, "lr_attn_decode_beside")
+    return True
+
+
 ATTN_DECODE_STATIC_MAX_BYTES = 32 << 20   # LR_ATTN_DECODE_STATIC_MAX_BYTES of include/ladder_hip.h
 
 
@@ -434,42 +461,53 @@ def advance(cur_token, next_token, pos, B, history=None, pos0=0):
            "lr_advance")
 
 
+def _ladder_model_desc(model, attention_workgroups: int = 0):
+    """lr_ladder_model_t for `model` (this rank's sizes), its device table of per-layer pointers, and the tensors
+    whose addresses they hold."""
+    cfg = model.config
+    dev = model.output.weight.device
+    rows, keep = [], []
+    for blk in model.layers:
+        ts = [blk.attention.wqkv.weight, blk.attention.wo.weight, blk.feed_forward.w1.weight,
+              blk.feed_forward.w2.weight, blk.attention_norm.weight, blk.ffn_norm.weight,
+              blk.attention.kv_cache.k_cache, blk.attention.kv_cache.v_cache]
+        for t in ts:
+            assert t.is_contiguous() and t.dtype == torch.bfloat16 and t.device == dev
+        keep.append(ts)
+        rows.append([t.data_ptr() for t in ts])
+    layer_table = torch.tensor(rows, dtype=torch.int64).to(dev)
+    keep += [model.tok_embeddings.weight, model.norm.weight, model.output.weight, model.freqs_cis]
+    desc = LadderModelDesc(
+        dim=cfg.dim, n_layer=cfg.n_layer, n_head=cfg.n_head_local, n_kv_head=cfg.n_kv_local, head_dim=cfg.head_dim,
+        ffn=cfg.ffn_local, out_rows=cfg.output_rows, vocab=cfg.vocab_size, smax=model.max_seq_length,
+        block_size=cfg.block_size, eps=cfg.norm_eps, attention_workgroups=attention_workgroups,
+        tok_embeddings=model.tok_embeddings.weight.data_ptr(),
+        norm=model.norm.weight.data_ptr(), output=model.output.weight.data_ptr(),
+        freqs_cis=model.freqs_cis.data_ptr(), layers_dev=layer_table.data_ptr())
+    return desc, layer_table, keep
+
+
+def _aligned_bytes(n: int, dev):
+    buf = torch.empty(n + 256, dtype=torch.uint8, device=dev)
+    off = (-buf.data_ptr()) % 256
+    return buf[off:off + n]
+
+
 class FusedLadderStep:
     """Device-side state of lr_ladder_decode_step for one model and batch size: the layer pointer
     table, the model descriptor and the (initialised) workspace.  Keeps references to every tensor
     whose address it handed to the library."""
 
     def __init__(self, model, batch: int, attention_workgroups: int = 0):
-        cfg = model.config
         dev = model.output.weight.device
-        rows = []
-        self._keep = []
-        for blk in model.layers:
-            ts = [blk.attention.wqkv.weight, blk.attention.wo.weight, blk.feed_forward.w1.weight,
-                  blk.feed_forward.w2.weight, blk.attention_norm.weight, blk.ffn_norm.weight,
-                  blk.attention.kv_cache.k_cache, blk.attention.kv_cache.v_cache]
-            for t in ts:
-                assert t.is_contiguous() and t.dtype == torch.bfloat16 and t.device == dev
-            self._keep.append(ts)
-            rows.append([t.data_ptr() for t in ts])
-        self.layer_table = torch.tensor(rows, dtype=torch.int64).to(dev)
-        self._keep += [model.tok_embeddings.weight, model.norm.weight, model.output.weight, model.freqs_cis]
-        self.desc = LadderModelDesc(
-            dim=cfg.dim, n_layer=cfg.n_layer, n_head=cfg.n_head_local, n_kv_head=cfg.n_kv_local, head_dim=cfg.head_dim,
-            ffn=cfg.ffn_local, out_rows=cfg.output_rows, vocab=cfg.vocab_size, smax=model.max_seq_length,
-            block_size=cfg.block_size, eps=cfg.norm_eps, attention_workgroups=attention_workgroups,
-            tok_embeddings=model.tok_embeddings.weight.data_ptr(),
-            norm=model.norm.weight.data_ptr(), output=model.output.weight.data_ptr(),
-            freqs_cis=model.freqs_cis.data_ptr(), layers_dev=self.layer_table.data_ptr())
+        self.desc, self.layer_table, self._keep = _ladder_model_desc(model, attention_workgroups)
         self.batch = batch
         lib = load()
         self.bytes = int(lib.lr_ladder_step_workspace_bytes(ctypes.byref(self.desc), batch))
         self.supported = self.bytes > 0
         self.workspace = None
         if self.supported:
-            self.workspace = torch.empty(self.bytes + 256, dtype=torch.uint8, device=dev)
-            off = (-self.workspace.data_ptr()) % 256
-            self.workspace = self.workspace[off:off + self.bytes]
+            self.workspace = _aligned_bytes(self.bytes, dev)
             self.reset()
 
     def reset(self):

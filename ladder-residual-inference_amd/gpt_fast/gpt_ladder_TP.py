@@ -140,6 +140,7 @@ class GPTLadder(GPTBase):
         # the weight-streaming kernel (q/k/v -- rotated and cached on the way out -- next to up/gate, which stores
         # silu(gate) * up directly), and so do its two output projections (wo next to w2)
         multi = side is None and 4 < ws.B <= 64 and not hasattr(self.layers[0].attention.wqkv, "scales")
+        beside = multi and ws.B <= 16
         for blk in self.layers:
             _hip.ladder_norms(ws.x, pending_a, pending_m, blk.attention_norm.weight, blk.ffn_norm.weight, ws.x, ws.xn,
                               ws.xn2, eps)
@@ -147,9 +148,19 @@ class GPTLadder(GPTBase):
                 kv = blk.attention.kv_cache
                 rope = _hip.rope_kv_epilogue(self.freqs_cis, pos, kv.k_cache, kv.v_cache, cfg.n_head_local,
                                              cfg.n_kv_local, cfg.head_dim)
-                _hip.linear_multi((ws.xn, blk.attention.wqkv.weight, ws.qkv, rope),
-                                  (ws.xn2, blk.feed_forward.w1.weight, ws.act, _hip.EPI_SWIGLU))
-                self._attention(ws, blk, pos, None, None, roped=True)
+                up_gate = (ws.xn2, blk.feed_forward.w1.weight, ws.act, _hip.EPI_SWIGLU)
+                if beside:
+                    # up to 16 rows the up/gate bands leave room for a second workgroup per CU: the attention's
+                    # items run in the same launch and wait for the KV cache behind the weight stream
+                    _hip.linear_multi((ws.xn, blk.attention.wqkv.weight, ws.qkv, rope))
+                    beside = _hip.attn_decode_beside(ws.qkv, kv.k_cache, kv.v_cache, pos, ws.y, ws.scratch, ws.B,
+                                                     cfg.n_head_local, cfg.n_kv_local, cfg.head_dim, up_gate)
+                    if not beside:
+                        _hip.linear_multi(up_gate)
+                        self._attention(ws, blk, pos, None, None, roped=True)
+                else:
+                    _hip.linear_multi((ws.xn, blk.attention.wqkv.weight, ws.qkv, rope), up_gate)
+                    self._attention(ws, blk, pos, None, None, roped=True)
                 _hip.linear_multi((ws.y, blk.attention.wo.weight, ws.a, _hip.EPI_NONE),
                                   (ws.act, blk.feed_forward.w2.weight, ws.m, _hip.EPI_NONE))
             elif side is not None:

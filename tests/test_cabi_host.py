@@ -75,6 +75,20 @@ def test_validation_precedes_any_device_work(lib):
     assert lib.lr_linear_multi(ptr, 1, 1, None) == E_SHAPE          # ldx < K
     one[0].ldx = 16
     assert lib.lr_linear_multi(ptr, 1, 1, None) == E_ALIGN
+    # attention beside a projection: attention arguments as lr_attn_decode, then what it has no kernel for
+    one[0] = _Projection(64, 8, 128, 256, 8, 8, 8, 0)
+
+    def beside(q, proj, M, epi=0, scratch_bytes=1 << 30):
+        one[0].epilogue = epi
+        return lib.lr_attn_decode_beside(q, 1024, 128, 256, 512, 1024, 1024, 4, 8, 1, 128, 64, 2048, scratch_bytes,
+                                         proj, M, None)
+
+    assert beside(None, ptr, 4) == E_NULL
+    assert beside(64, None, 4) == E_NULL
+    assert beside(64, ptr, 0) == E_SHAPE
+    assert beside(64, ptr, 17) == -4                                # the 16-row band only
+    assert beside(64, ptr, 4, epi=2) == -4                          # a projection that writes the cache
+    assert beside(64, ptr, 4, scratch_bytes=16) == E_SHAPE
     assert lib.lr_ladder_decode_step(None, 1, None, None, None, 0, None, 0, None, None, 0, 0, 0, None, 0, None) == E_NULL
     assert lib.lr_ladder_step_workspace_bytes(None, 1) == 0
 

@@ -476,6 +476,59 @@ def test_attn_decode(hip, B, Hq, Hkv, hd, Smax, pos):
     assert_close_ulp(y, want, max_frac=0.03, what="attn_decode")
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,hd,Smax,pos,D,I,epi_swiglu", [
+    (8, 8, 1, 128, 2176, 2100, 1024, 456, True),     # the 70B rank shard's heads at batch 8
+    (16, 32, 8, 128, 1100, 1024, 512, 1000, True),   # Ladder-8B's heads at batch 16
+    (5, 4, 2, 64, 300, 0, 264, 72, True),            # first position: one key per sequence
+    (16, 8, 8, 64, 520, 519, 136, 4100, False),      # one q head per kv head, a plain projection beside it
+    (1, 2, 1, 128, 64, 63, 64, 16, True),
+])
+def test_attn_decode_beside_equals_the_two_calls(hip, B, Hq, Hkv, hd, Smax, pos, D, I, epi_swiglu):
+    """Attention items and projection bands in one grid: same bits as lr_attn_decode, then lr_linear_multi."""
+    q = rnd(B, (Hq + 2 * Hkv) * hd, seed=50)         # q is the head of the fused q/k/v row, as in a decode step
+    kc, vc = rnd(B, Hkv, Smax, hd, seed=51), rnd(B, Hkv, Smax, hd, seed=52)
+    kc[:, :, pos + 1:] = 7.0
+    vc[:, :, pos + 1:] = -9.0
+    p = torch.tensor([pos], dtype=torch.int32, device=DEV)
+    x = rnd(B, D, seed=53)
+    w = rnd(2 * I if epi_swiglu else I, D, seed=54, scale=0.05)
+    epi = hip.EPI_SWIGLU if epi_swiglu else hip.EPI_NONE
+    nscr = hip.attn_decode_scratch_bytes(B, Hq, hd, Smax) // 4
+    y, out = [torch.zeros(B, Hq * hd, dtype=BF, device=DEV) for _ in range(2)], \
+        [torch.zeros(B, I, dtype=BF, device=DEV) for _ in range(2)]
+    scratch = [torch.zeros(nscr, dtype=torch.float32, device=DEV) for _ in range(2)]
+    hip.attn_decode(q, kc, vc, p, y[0], scratch[0], B, Hq, Hkv, hd)
+    hip.linear_multi((x, w, out[0], epi))
+    assert hip.attn_decode_beside(q, kc, vc, p, y[1], scratch[1], B, Hq, Hkv, hd, (x, w, out[1], epi))
+    assert torch.equal(y[1], y[0]) and torch.equal(out[1], out[0])
+    mask = (torch.arange(Smax, device=DEV) <= pos).view(1, Smax)
+    want = O.sdpa_math(q[:, :Hq * hd].reshape(B, 1, Hq, hd).transpose(1, 2), kc, vc, mask).transpose(1, 2)
+    assert_close_ulp(y[1], want.reshape(B, Hq * hd), max_frac=0.03, what="attn_decode_beside")
+
+
+def test_attn_decode_beside_declines_what_it_has_no_kernel_for(hip):
+    """More than 16 rows, 16 q heads per kv head, or a projection that writes the cache: False, nothing launched."""
+    def run(B, Hq, Hkv, epi=None):
+        hd, Smax, D, I = 128, 64, 64, 16
+        q = rnd(B, Hq * hd, seed=55)
+        kc, vc = rnd(B, Hkv, Smax, hd, seed=56), rnd(B, Hkv, Smax, hd, seed=57)
+        p = torch.tensor([3], dtype=torch.int32, device=DEV)
+        y = torch.full((B, Hq * hd), 5.0, dtype=BF, device=DEV)
+        N = (Hq + 2 * Hkv) * hd if epi is not None else I
+        out = torch.full((B, N), 5.0, dtype=BF, device=DEV)
+        scratch = torch.zeros(hip.attn_decode_scratch_bytes(B, Hq, hd, Smax) // 4, dtype=torch.float32, device=DEV)
+        if epi is not None:
+            epi = hip.rope_kv_epilogue(O.rope_table(64, hd, 10000.0, BF).to(DEV), p, kc, vc, Hq, Hkv, hd)
+        ok = hip.attn_decode_beside(q, kc, vc, p, y, scratch, B, Hq, Hkv, hd,
+                                    (rnd(B, D, seed=58), rnd(N, D, seed=59), out, hip.EPI_NONE if epi is None else epi))
+        torch.cuda.synchronize()
+        return ok, bool((y == 5.0).all()) and bool((out == 5.0).all())
+    assert run(17, 8, 1) == (False, True)
+    assert run(4, 16, 1) == (False, True)
+    assert run(4, 8, 1, epi="rope") == (False, True)
+    assert run(4, 8, 1)[0] is True
+
+
 @pytest.mark.parametrize("B,S,Hq,Hkv,hd,Smax,start", [
     (1, 128, 8, 1, 128, 136, 0), (2, 100, 4, 2, 64, 160, 0), (1, 300, 8, 1, 128, 512, 100), (1, 2048, 8, 1, 128, 2176, 0),
     (3, 65, 32, 8, 64, 72, 0),
