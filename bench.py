@@ -109,7 +109,7 @@ def decode_run(bm, model, prompt, B, T, K, W):
     return ms, first, dg
 
 
-def extra_batched(bm, model, prompt, T, batches=(8, 64), K=32, W=5):
+def extra_batched(bm, model, prompt, T, batches=(4, 8, 64), K=32, W=5):
     """The headline shard at the other batch sizes of the benchmark set (per-op kernels)."""
     cfg = model.config
     out = []

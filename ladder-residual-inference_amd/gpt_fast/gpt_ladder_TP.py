@@ -136,10 +136,12 @@ class GPTLadder(GPTBase):
             if side is None or side.device != main.device:
                 side = self._side_stream = torch.cuda.Stream(device=main.device)
         pending_a = pending_m = None
-        # decode batches of 5 to 64 rows on bf16 weights: the block's two input projections share one launch of
+        # decode batches of up to 64 rows on bf16 weights: the block's two input projections share one launch of
         # the weight-streaming kernel (q/k/v -- rotated and cached on the way out -- next to up/gate, which stores
-        # silu(gate) * up directly), and so do its two output projections (wo next to w2)
-        multi = side is None and 4 < ws.B <= 64 and not hasattr(self.layers[0].attention.wqkv, "scales")
+        # silu(gate) * up directly), and so do its two output projections (wo next to w2).  Also below 5 rows,
+        # where single projections go to the matrix-vector kernel: five or six launches per block instead of nine
+        # weigh more than the kernel (70B rank shard, ms per step: batch 1 4.9 / 5.5, batch 4 5.0 / 8.3)
+        multi = side is None and ws.B <= 64 and not hasattr(self.layers[0].attention.wqkv, "scales")
         beside = multi and ws.B <= 16
         for blk in self.layers:
             _hip.ladder_norms(ws.x, pending_a, pending_m, blk.attention_norm.weight, blk.ffn_norm.weight, ws.x, ws.xn,
