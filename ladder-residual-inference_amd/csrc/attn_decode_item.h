@@ -4,6 +4,7 @@
 // ---- how the valid keys are cut into chunks (one workgroup item per chunk, kv head and sequence).
 //      A chunk never exceeds ATT_CHUNK keys: the item then requests all of its K and V rows at once.
 constexpr int ATT_CHUNK = 256;
+constexpr int ATT_NCU = 256;  // CUs of the MI355X
 
 static inline int attn_nsplit_cap(int Smax) {
   const int by_len = (Smax + ATT_CHUNK - 1) / ATT_CHUNK;
@@ -18,7 +19,20 @@ static inline int attn_pick_nsplit(int B, int Hkv, int Smax) {
   const int by_len = (Smax + ATT_CHUNK - 1) / ATT_CHUNK;
   if (n < by_len) n = by_len;
   if (n < 1) n = 1;
-  return n > cap ? cap : n;
+  if (n > cap) n = cap;
+  // With more items than CUs the slowest CU sets the time: among the neighbouring chunk counts take the one
+  // whose items fill whole rounds of the 256 CUs best (64 sequences: 12 chunks = 768 items instead of 9 = 576).
+  if ((int64_t)n * B * Hkv >= ATT_NCU) {
+    int best = n;
+    int64_t best_num = 0, best_den = 1;  // padded / real items of the best candidate
+    const int lo = n - 3 > by_len ? n - 3 : by_len, hi = n + 3 < cap ? n + 3 : cap;
+    for (int c = lo < 1 ? 1 : lo; c <= hi; ++c) {
+      const int64_t items = (int64_t)c * B * Hkv, padded = (items + ATT_NCU - 1) / ATT_NCU * ATT_NCU;
+      if (best_num == 0 || padded * best_den < best_num * items) { best = c; best_num = padded; best_den = items; }
+    }
+    n = best;
+  }
+  return n;
 }
 
 // LDS row length of the score buffer: whole 16-key tiles, plus 4 so that the 16 heads a tile's scores are
