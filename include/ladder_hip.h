@@ -159,7 +159,8 @@ int lr_linear_swiglu_out(const void* x, int64_t ldx, const void* w, void* y, int
  * the attention's all-reduce with the MLP for the same reason); the two halves must be independent of each
  * other.  Same bits as lr_attn_decode(q, ..., y) followed by lr_linear_multi(projection, 1, M).
  * Arguments as there.  LR_E_UNSUPPORTED (nothing launched): M > 16, an LR_EPI_ROPE_KV projection (it would write
- * the cache the attention reads), more than 8 q heads per kv head -- the caller then makes the two calls. */
+ * the cache the attention reads), q heads per kv head other than 1, 2, 4, 8, 16 -- the caller then makes the two
+ * calls. */
 int lr_attn_decode_beside(const void* q, int64_t ldq, const void* k_cache, const void* v_cache, const int32_t* pos,
                           void* y, int64_t ldy, int B, int Hq, int Hkv, int hd, int Smax, void* scratch,
                           size_t scratch_bytes, const lr_projection_t* projection, int M, lr_stream_t stream);

@@ -41,7 +41,8 @@ __host__ __device__ constexpr int attn_sc_ld(int chunk_max) { return ((chunk_max
 
 // One (split, kv head, sequence) item of the split-KV decode attention, by 256 lanes (4 waves): scores,
 // softmax statistics and the un-normalised P.V of keys [k0, k1) (at most ATT_CHUNK) for all G q heads of
-// the kv head.  `smem`: attn_item_lds_floats<HD, G>(chunk_max) floats of LDS.
+// the kv head.  `smem`: attn_item_lds_floats<HD, G>(chunk_max) floats of LDS.  (A kv head with more q heads than
+// an instantiation takes can be served as kv_share groups of G: every head's result is the same either way.)
 //
 // Every K and V row of the chunk is requested before anything else -- whole rows, 1 KiB contiguous per
 // wave instruction, up to 32 KiB per wave in flight -- so the item costs one memory round trip.  Scores
@@ -60,7 +61,7 @@ __device__ __forceinline__ void attn_partial_item(const u16* __restrict__ q, int
                                                   const u16* __restrict__ vc, const int32_t* __restrict__ pos_ptr,
                                                   float* __restrict__ o_part, float* __restrict__ ml_part, int Hkv,
                                                   int Smax, int nsplit, int chunk_max, int split, int kvh, int b,
-                                                  float* __restrict__ smem) {
+                                                  float* __restrict__ smem, int kv_share = 1) {
   static_assert(G <= 16, "the q heads of a kv head are the 16 columns of one matrix-core tile");
   constexpr int LPK = HD / 8;    // lanes that share one key row (8 elements each)
   constexpr int KPW = 64 / LPK;  // keys per wave instruction
@@ -97,8 +98,9 @@ __device__ __forceinline__ void attn_partial_item(const u16* __restrict__ q, int
   }
 
   const int kl = lane / LPK, dl = (lane % LPK) * 8;
-  const u16* kbase = kc + ((int64_t)b * Hkv + kvh) * Smax * HD;
-  const u16* vbase = vc + ((int64_t)b * Hkv + kvh) * Smax * HD;
+  // kv_share > 1: `Hkv` and `kvh` count groups of G q heads, kv_share of them on one head of the cache
+  const u16* kbase = kc + ((int64_t)b * (Hkv / kv_share) + kvh / kv_share) * Smax * HD;
+  const u16* vbase = vc + ((int64_t)b * (Hkv / kv_share) + kvh / kv_share) * Smax * HD;
   const float scale = rsqrtf((float)HD);
   // wave w owns the 16-key tiles w, w + 4, ...; instruction i of a tile covers keys i * KPW .. + KPW
   uint4 kr[TPW][NI], vr[TPW][NI];

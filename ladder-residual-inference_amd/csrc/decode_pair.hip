@@ -26,7 +26,8 @@ struct AttnItems {
   const int32_t* pos;
   float* o_part;
   float* ml_part;
-  int Hkv, Smax, nsplit, chunk_max;
+  int Hkv, Smax, nsplit, chunk_max;  // Hkv: groups of G q heads (kv_share of them per head of the cache)
+  int kv_share;
   int n_items;  // nsplit * Hkv * B: the first workgroups of the grid
 };
 
@@ -39,7 +40,8 @@ __global__ __launch_bounds__(256) void k_attn_beside_band(const AttnItems a, con
   if (wg < a.n_items) {
     const int split = wg % a.nsplit, rest = wg / a.nsplit;
     attn_partial_item<HD, G>(a.q, a.ldq, a.kc, a.vc, a.pos, a.o_part, a.ml_part, a.Hkv, a.Smax, a.nsplit,
-                             a.chunk_max, split, rest % a.Hkv, rest / a.Hkv, reinterpret_cast<float*>(pair_smem));
+                             a.chunk_max, split, rest % a.Hkv, rest / a.Hkv, reinterpret_cast<float*>(pair_smem),
+                             a.kv_share);
   } else {
     stream_band<PAIR_MT, PAIR_UNITS>(p, M, wg - a.n_items, reinterpret_cast<u16*>(pair_smem));
   }
@@ -82,16 +84,23 @@ extern "C" int lr_attn_decode_beside(const void* q, int64_t ldq, const void* k_c
   Proj p;
   const int rc = sb_fill_projection(*proj, p);
   if (rc != LR_OK) return rc;
-  const int G = Hq / Hkv;
+  int G = Hq / Hkv;
   AttnItems a;
+  a.kv_share = 1;
   a.q = (const u16*)q; a.ldq = ldq; a.kc = (const u16*)k_cache; a.vc = (const u16*)v_cache; a.pos = pos;
-  a.Hkv = Hkv; a.Smax = Smax;
-  a.nsplit = attn_pick_nsplit(B, Hkv, Smax);
+  a.Smax = Smax;
+  a.nsplit = attn_pick_nsplit(B, Hkv, Smax);  // the chunks of lr_attn_decode
+  if (G == 16) {
+    // 16 q heads per kv head need the whole register file (one workgroup per CU): two groups of 8 instead
+    G = 8;
+    a.kv_share = 2;
+  }
+  a.Hkv = Hkv * a.kv_share;
   a.chunk_max = ((Smax + a.nsplit - 1) / a.nsplit + 3) & ~3;
   a.o_part = (float*)scratch;
   a.ml_part = a.o_part + (size_t)B * Hq * a.nsplit * hd;
-  if ((int64_t)a.nsplit * Hkv * B > 0x3fffffff) return LR_E_UNSUPPORTED;
-  a.n_items = a.nsplit * Hkv * B;
+  if ((int64_t)a.nsplit * a.Hkv * B > 0x3fffffff) return LR_E_UNSUPPORTED;
+  a.n_items = a.nsplit * a.Hkv * B;
   if (!((hd == 128 || hd == 64) && (G == 1 || G == 2 || G == 4 || G == 8))) return LR_E_UNSUPPORTED;
   const int ncu = sb_num_cus();
   if (ncu < 1) return LR_E_LAUNCH;

@@ -481,6 +481,8 @@ def test_attn_decode(hip, B, Hq, Hkv, hd, Smax, pos):
     (16, 32, 8, 128, 1100, 1024, 512, 1000, True),   # Ladder-8B's heads at batch 16
     (5, 4, 2, 64, 300, 0, 264, 72, True),            # first position: one key per sequence
     (16, 8, 8, 64, 520, 519, 136, 4100, False),      # one q head per kv head, a plain projection beside it
+    (16, 16, 1, 128, 4224, 4100, 512, 456, True),    # the 405B rank shard's heads: 16 q heads as two groups of 8
+    (3, 32, 2, 128, 200, 150, 264, 64, True),
     (1, 2, 1, 128, 64, 63, 64, 16, True),
 ])
 def test_attn_decode_beside_equals_the_two_calls(hip, B, Hq, Hkv, hd, Smax, pos, D, I, epi_swiglu):
@@ -507,7 +509,7 @@ def test_attn_decode_beside_equals_the_two_calls(hip, B, Hq, Hkv, hd, Smax, pos,
 
 
 def test_attn_decode_beside_declines_what_it_has_no_kernel_for(hip):
-    """More than 16 rows, 16 q heads per kv head, or a projection that writes the cache: False, nothing launched."""
+    """More than 16 rows, 32 q heads per kv head, or a projection that writes the cache: False, nothing launched."""
     def run(B, Hq, Hkv, epi=None):
         hd, Smax, D, I = 128, 64, 64, 16
         q = rnd(B, Hq * hd, seed=55)
@@ -524,7 +526,7 @@ def test_attn_decode_beside_declines_what_it_has_no_kernel_for(hip):
         torch.cuda.synchronize()
         return ok, bool((y == 5.0).all()) and bool((out == 5.0).all())
     assert run(17, 8, 1) == (False, True)
-    assert run(4, 16, 1) == (False, True)
+    assert run(4, 32, 1) == (False, True)
     assert run(4, 8, 1, epi="rope") == (False, True)
     assert run(4, 8, 1)[0] is True
 
