@@ -22,7 +22,8 @@ static inline int attn_pick_nsplit(int B, int Hkv, int Smax) {
   if (n > cap) n = cap;
   // With more items than CUs the slowest CU sets the time: among the neighbouring chunk counts take the one
   // whose items fill whole rounds of the 256 CUs best (64 sequences: 12 chunks = 768 items instead of 9 = 576).
-  if ((int64_t)n * B * Hkv >= ATT_NCU) {
+  // (beyond four rounds the gain is smaller than the cost of more chunks to merge)
+  if ((int64_t)n * B * Hkv >= ATT_NCU && (int64_t)n * B * Hkv < 4 * ATT_NCU) {
     int best = n;
     int64_t best_num = 0, best_den = 1;  // padded / real items of the best candidate
     const int lo = n - 3 > by_len ? n - 3 : by_len, hi = n + 3 < cap ? n + 3 : cap;
