@@ -180,6 +180,25 @@ size_t lr_linear_fp8_scratch_bytes(int M, int N, int K);
 int lr_linear_fp8(const void* x, int64_t ldx, const void* w8, const void* scales, void* y, int64_t ldy, int M, int N,
                   int K, void* scratch, size_t scratch_bytes, lr_stream_t stream);
 
+/* lr_linear_multi for weight-only e4m3 projections, M <= 8 input rows (LR_E_UNSUPPORTED beyond): one or two
+ * projections per launch, per projection y = F.linear(x, w8.to(bf16)) * scales as lr_linear_fp8 computes it
+ * (same bits), then the epilogue on those values -- LR_EPI_SWIGLU: w8 holds [up; gate] rows, y[M, N / 2] =
+ * bf16( bf16(silu(g)) * u ) (utils.py:145-148); LR_EPI_ROPE_KV: the q/k/v projection of a decode step, finished
+ * as lr_rope_kv_write would (utils.py:193-198, :50-59).  What the per-op decode step of a quantised ladder block
+ * needs in two launches: {q/k/v next to up/gate} and {wo next to w2} (gpt_ladder_TP.py:323-349).  K % 16 == 0. */
+typedef struct lr_projection_fp8 {
+  const void* x; /* [M, K] bf16, row stride ldx */
+  int64_t ldx;
+  const void* w8;     /* [N, K] float8_e4m3fn, dense */
+  const void* scales; /* [N] bf16 */
+  void* y;            /* [M, N] (or [M, N / 2]) bf16, row stride ldy */
+  int64_t ldy;
+  int32_t N, K;
+  int32_t epilogue;
+  const lr_rope_kv_t* rope; /* LR_EPI_ROPE_KV only, else ignored; read during the call */
+} lr_projection_fp8_t;
+int lr_linear_fp8_multi(const lr_projection_fp8_t* projections, int n_projections, int M, lr_stream_t stream);
+
 /* out[r, i] = bf16( bf16(silu(h[r, I + i])) * h[r, i] ),  h [rows, 2I] = [u | g] (row stride ldh).
  * F.silu(g) * u after chunk(2), utils.py:147-148 and :386. */
 int lr_swiglu(const void* h, int64_t ldh, void* out, int rows, int I, lr_stream_t stream);

@@ -29,6 +29,7 @@ _PROTOS = {
     "lr_linear_swiglu_out": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p,
                                      c_size_t, c_void_p]),
     "lr_linear_fp8_scratch_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "lr_linear_fp8_multi": (c_int, [c_void_p, c_int, c_int, c_void_p]),
     "lr_linear_fp8": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p,
                               c_size_t, c_void_p]),
     "lr_swiglu": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_int, c_void_p]),
@@ -241,6 +242,36 @@ def _projection_array(projections):
         arr[i] = _Projection(_dev(x), ldx, _dev(w), _dev(out), ldy, N, K, epi,
                              ctypes.pointer(rope) if rope is not None else None)
     return arr, M, keep
+
+
+class _ProjectionFp8(ctypes.Structure):
+    """lr_projection_fp8_t of include/ladder_hip.h."""
+    _fields_ = [("x", c_void_p), ("ldx", c_int64), ("w8", c_void_p), ("scales", c_void_p), ("y", c_void_p),
+                ("ldy", c_int64), ("N", c_int32), ("K", c_int32), ("epilogue", c_int32), ("rope", ctypes.POINTER(_RopeKv))]
+
+
+def linear_fp8_multi(*projections):
+    """linear_multi for weight-only e4m3 projections of the same M <= 8 rows (lr_linear_fp8_multi).  Each projection
+    is (x [M, K], w8 [N, K] float8_e4m3fn, scales [N], out, epilogue), epilogue as in linear_multi."""
+    arr = (_ProjectionFp8 * len(projections))()
+    M = None
+    keep = []
+    for i, (x, w8, scales, out, epi) in enumerate(projections):
+        rope = None
+        if isinstance(epi, _RopeKv):
+            rope, epi = epi, EPI_ROPE_KV
+            keep.append(rope)
+        m, K, ldx = _rows_ld(x)
+        N, Kw = w8.shape
+        Mo, No, ldy = _rows_ld(out)
+        assert w8.dtype == torch.float8_e4m3fn and w8.is_contiguous() and w8.is_cuda and Kw == K
+        assert scales.dtype == torch.bfloat16 and scales.numel() == N and scales.is_contiguous()
+        assert Mo == m and No == (N // 2 if epi == EPI_SWIGLU else N), (x.shape, w8.shape, out.shape, epi)
+        assert M is None or M == m
+        M = m
+        arr[i] = _ProjectionFp8(_dev(x), ldx, w8.data_ptr(), _dev(scales), _dev(out), ldy, N, K, epi,
+                                ctypes.pointer(rope) if rope is not None else None)
+    _check(load().lr_linear_fp8_multi(ctypes.cast(arr, c_void_p), len(projections), M, _stream()), "lr_linear_fp8_multi")
 
 
 def linear_fp8(x: torch.Tensor, w8: torch.Tensor, scales: torch.Tensor, out: torch.Tensor):

@@ -141,8 +141,11 @@ class GPTLadder(GPTBase):
         # silu(gate) * up directly), and so do its two output projections (wo next to w2).  Also below 5 rows,
         # where single projections go to the matrix-vector kernel: five or six launches per block instead of nine
         # weigh more than the kernel (70B rank shard, ms per step: batch 1 4.9 / 5.5, batch 4 5.0 / 8.3)
-        multi = side is None and ws.B <= 64 and not hasattr(self.layers[0].attention.wqkv, "scales")
+        fp8 = hasattr(self.layers[0].attention.wqkv, "scales")
+        multi = side is None and ws.B <= 64 and not fp8
         beside = multi and ws.B <= 16
+        # weight-only e4m3 projections, up to 8 rows: the same two launches per block from the fp8 matrix-vector kernel
+        multi8 = side is None and fp8 and ws.B <= 8
         for blk in self.layers:
             _hip.ladder_norms(ws.x, pending_a, pending_m, blk.attention_norm.weight, blk.ffn_norm.weight, ws.x, ws.xn,
                               ws.xn2, eps)
@@ -165,6 +168,15 @@ class GPTLadder(GPTBase):
                     self._attention(ws, blk, pos, None, None, roped=True)
                 _hip.linear_multi((ws.y, blk.attention.wo.weight, ws.a, _hip.EPI_NONE),
                                   (ws.act, blk.feed_forward.w2.weight, ws.m, _hip.EPI_NONE))
+            elif multi8:
+                att, ff, kv = blk.attention, blk.feed_forward, blk.attention.kv_cache
+                rope = _hip.rope_kv_epilogue(self.freqs_cis, pos, kv.k_cache, kv.v_cache, cfg.n_head_local,
+                                             cfg.n_kv_local, cfg.head_dim)
+                _hip.linear_fp8_multi((ws.xn, att.wqkv.weight, att.wqkv.scales, ws.qkv, rope),
+                                      (ws.xn2, ff.w1.weight, ff.w1.scales, ws.act, _hip.EPI_SWIGLU))
+                self._attention(ws, blk, pos, None, None, roped=True)
+                _hip.linear_fp8_multi((ws.y, att.wo.weight, att.wo.scales, ws.a, _hip.EPI_NONE),
+                                      (ws.act, ff.w2.weight, ff.w2.scales, ws.m, _hip.EPI_NONE))
             elif side is not None:
                 side.wait_stream(main)
                 with torch.cuda.stream(side):

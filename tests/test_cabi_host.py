@@ -89,6 +89,18 @@ def test_validation_precedes_any_device_work(lib):
     assert beside(64, ptr, 17) == -4                                # the 16-row band only
     assert beside(64, ptr, 4, epi=2) == -4                          # a projection that writes the cache
     assert beside(64, ptr, 4, scratch_bytes=16) == E_SHAPE
+    from gpt_fast._hip import _ProjectionFp8
+    one8 = (_ProjectionFp8 * 1)(_ProjectionFp8(64, 16, 128, 192, 256, 8, 8, 16, 0))
+    ptr8 = ctypes.cast(one8, ctypes.c_void_p)
+    assert lib.lr_linear_fp8_multi(None, 1, 1, None) == E_NULL
+    assert lib.lr_linear_fp8_multi(ptr8, 1, 9, None) == -4            # the matrix-vector kernel takes up to 8 rows
+    assert lib.lr_linear_fp8_multi(ptr8, 3, 1, None) == E_SHAPE
+    one8[0].K = 24                                                    # 16 weights per lane and load
+    assert lib.lr_linear_fp8_multi(ptr8, 1, 1, None) == E_SHAPE       # ldx < K
+    one8[0].ldx = 24
+    assert lib.lr_linear_fp8_multi(ptr8, 1, 1, None) == E_ALIGN
+    one8[0].K, one8[0].ldx, one8[0].scales = 16, 16, None
+    assert lib.lr_linear_fp8_multi(ptr8, 1, 1, None) == E_NULL
     assert lib.lr_ladder_decode_step(None, 1, None, None, None, 0, None, 0, None, None, 0, 0, 0, None, 0, None) == E_NULL
     assert lib.lr_ladder_step_workspace_bytes(None, 1) == 0
 

@@ -431,6 +431,50 @@ def test_linear_fp8(hip, M, N, K):
     assert_close_ulp(y, exact, max_ulp=2, max_frac=0.4, what="fp8 linear vs fp64")
 
 
+@pytest.mark.parametrize("M,D,Hq,Hkv,hd,I", [(1, 8192, 8, 1, 128, 3584), (8, 8192, 8, 1, 128, 3584), (3, 4096, 32, 8, 128, 1000),
+                                             (5, 2048, 4, 2, 64, 72), (2, 1040, 2, 2, 64, 17), (4, 64, 1, 1, 8, 8)])
+def test_linear_fp8_multi_equals_the_separate_calls(hip, M, D, Hq, Hkv, hd, I):
+    """Two e4m3 projections per launch with their epilogues: q/k/v rotated and cached as lr_linear_fp8 followed by
+    lr_rope_kv_write leaves them, up/gate as lr_linear_fp8 followed by lr_swiglu, plain projections as lr_linear_fp8
+    -- bit for bit; rows (2p, 2p + 1) and (p, p + I) of one wave, K below and above the K-split thresholds."""
+    Smax, block, pos_value = 40, 64, 23
+    NQ = (Hq + 2 * Hkv) * hd
+    xa, xb = rnd(M, D, seed=60), rnd(M, D, seed=61)
+    wq, sq = O.quantize_fp8_rowwise(rnd(NQ, D, seed=62, scale=0.03, dtype=torch.float32), BF)
+    w1, s1 = O.quantize_fp8_rowwise(rnd(2 * I, D, seed=63, scale=0.03, dtype=torch.float32), BF)
+    table = O.rope_table(block, hd, 10000.0, BF).to(DEV)
+    pos = torch.tensor([pos_value], dtype=torch.int32, device=DEV)
+    kc = [rnd(M, Hkv, Smax, hd, seed=64) for _ in range(2)]
+    vc = [rnd(M, Hkv, Smax, hd, seed=65) for _ in range(2)]
+    # separate calls
+    q_ref = torch.empty(M, NQ, dtype=BF, device=DEV)
+    hip.linear_fp8(xa, wq, sq, q_ref)
+    kv_proj = q_ref[:, Hq * hd:].clone()
+    hip.rope_kv_write(q_ref, table, False, pos, kc[0], vc[0], M, 1, Hq, Hkv, hd)
+    h = torch.empty(M, 2 * I, dtype=BF, device=DEV)
+    hip.linear_fp8(xb, w1, s1, h)
+    act_ref = F.silu(h[:, I:]) * h[:, :I]
+    # one launch
+    q = torch.empty(M, NQ, dtype=BF, device=DEV)
+    act = torch.full((M, I), 3.0, dtype=BF, device=DEV)
+    hip.linear_fp8_multi((xa, wq, sq, q, hip.rope_kv_epilogue(table, pos, kc[1], vc[1], Hq, Hkv, hd)),
+                         (xb, w1, s1, act, hip.EPI_SWIGLU))
+    assert torch.equal(q[:, :Hq * hd], q_ref[:, :Hq * hd]) and torch.equal(q[:, Hq * hd:], kv_proj)
+    assert torch.equal(kc[1], kc[0]) and torch.equal(vc[1], vc[0])
+    assert torch.equal(act, act_ref)
+    # plain projections, one of them with an odd number of rows
+    wo, so = O.quantize_fp8_rowwise(rnd(D + 1, Hq * hd, seed=66, scale=0.03, dtype=torch.float32), BF) if (Hq * hd) % 16 == 0 \
+        else (None, None)
+    if wo is not None:
+        y = rnd(M, Hq * hd, seed=67)
+        a_ref, a = torch.empty(M, D + 1, dtype=BF, device=DEV), torch.zeros(M, D + 9, dtype=BF, device=DEV)
+        hip.linear_fp8(y, wo, so, a_ref)
+        m_ref, m = torch.empty(M, NQ, dtype=BF, device=DEV), torch.empty(M, NQ, dtype=BF, device=DEV)
+        hip.linear_fp8(xa, wq, sq, m_ref)
+        hip.linear_fp8_multi((y, wo, so, a[:, :D + 1], hip.EPI_NONE), (xa, wq, sq, m, hip.EPI_NONE))
+        assert torch.equal(a[:, :D + 1], a_ref) and bool((a[:, D + 1:] == 0).all()) and torch.equal(m, m_ref)
+
+
 def test_rope_kv_write_position_out_of_range_sets_the_error_word(hip):
     """Positions beyond the cache or the RoPE table: the row is left alone, nothing lands in the cache and the
     per-device error word becomes LR_DEV_POS_RANGE (the reference raises an index error, utils.py:55)."""
