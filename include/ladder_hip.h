@@ -180,9 +180,10 @@ size_t lr_linear_fp8_scratch_bytes(int M, int N, int K);
 int lr_linear_fp8(const void* x, int64_t ldx, const void* w8, const void* scales, void* y, int64_t ldy, int M, int N,
                   int K, void* scratch, size_t scratch_bytes, lr_stream_t stream);
 
-/* lr_linear_multi for weight-only e4m3 projections, M <= 8 input rows (LR_E_UNSUPPORTED beyond): one or two
- * projections per launch, per projection y = F.linear(x, w8.to(bf16)) * scales as lr_linear_fp8 computes it
- * (same bits), then the epilogue on those values -- LR_EPI_SWIGLU: w8 holds [up; gate] rows, y[M, N / 2] =
+/* lr_linear_multi for weight-only e4m3 projections, M <= 16 input rows (LR_E_UNSUPPORTED beyond): one or two
+ * projections per launch, per projection y = F.linear(x, w8.to(bf16)) * scales with lr_linear_fp8's two roundings
+ * (M == 1: the matrix-vector kernel, lr_linear_fp8's bits; from 2 rows on the matrix-core bands of lr_linear_multi
+ * with the weights expanded on their way through LDS), then the epilogue on those values -- LR_EPI_SWIGLU: w8 holds [up; gate] rows, y[M, N / 2] =
  * bf16( bf16(silu(g)) * u ) (utils.py:145-148); LR_EPI_ROPE_KV: the q/k/v projection of a decode step, finished
  * as lr_rope_kv_write would (utils.py:193-198, :50-59).  What the per-op decode step of a quantised ladder block
  * needs in two launches: {q/k/v next to up/gate} and {wo next to w2} (gpt_ladder_TP.py:323-349).  K % 16 == 0. */
@@ -198,6 +199,16 @@ typedef struct lr_projection_fp8 {
   const lr_rope_kv_t* rope; /* LR_EPI_ROPE_KV only, else ignored; read during the call */
 } lr_projection_fp8_t;
 int lr_linear_fp8_multi(const lr_projection_fp8_t* projections, int n_projections, int M, lr_stream_t stream);
+
+/* lr_attn_decode_beside with a weight-only e4m3 projection (one lr_projection_fp8_t of lr_linear_fp8_multi) in
+ * place of the bf16 one: the quantised ladder block's up/gate projection next to its attention.  Same bits as
+ * lr_attn_decode followed by lr_linear_fp8_multi(projection, 1, M).  LR_E_UNSUPPORTED (nothing launched): M == 1
+ * (lr_linear_fp8_multi uses the matrix-vector kernel there) or M > 16, an LR_EPI_ROPE_KV projection, q heads per
+ * kv head other than 1, 2, 4, 8, 16. */
+int lr_attn_decode_beside_fp8(const void* q, int64_t ldq, const void* k_cache, const void* v_cache,
+                              const int32_t* pos, void* y, int64_t ldy, int B, int Hq, int Hkv, int hd, int Smax,
+                              void* scratch, size_t scratch_bytes, const lr_projection_fp8_t* projection, int M,
+                              lr_stream_t stream);
 
 /* out[r, i] = bf16( bf16(silu(h[r, I + i])) * h[r, i] ),  h [rows, 2I] = [u | g] (row stride ldh).
  * F.silu(g) * u after chunk(2), utils.py:147-148 and :386. */

@@ -13,6 +13,9 @@
 // attention's chunks stays a launch of its own: done inside this one by whoever stores the last
 // chunk of a kv head (chunk results written through to the memory side, one ticket per kv head),
 // it became the tail of the grid instead of hiding in it (0.4 ms per step slower at batch 8 and 16).
+//
+// lr_attn_decode_beside_fp8: the same grid with the e4m3 variant of the band (weight-only quantised models,
+// 2 to 16 rows).
 #include "attn_decode_item.h"
 #include "stream_band.h"
 
@@ -33,7 +36,7 @@ struct AttnItems {
 
 constexpr int PAIR_MT = 16, PAIR_UNITS = 2;
 
-template <int HD, int G>
+template <int HD, int G, bool W8>
 __global__ __launch_bounds__(256) void k_attn_beside_band(const AttnItems a, const Proj p, const int M) {
   extern __shared__ __attribute__((aligned(16))) unsigned char pair_smem[];
   const int wg = blockIdx.x;
@@ -43,32 +46,31 @@ __global__ __launch_bounds__(256) void k_attn_beside_band(const AttnItems a, con
                              a.chunk_max, split, rest % a.Hkv, rest / a.Hkv, reinterpret_cast<float*>(pair_smem),
                              a.kv_share);
   } else {
-    stream_band<PAIR_MT, PAIR_UNITS>(p, M, wg - a.n_items, reinterpret_cast<u16*>(pair_smem));
+    stream_band<PAIR_MT, PAIR_UNITS, W8>(p, M, wg - a.n_items, reinterpret_cast<u16*>(pair_smem));
   }
 }
 
-template <int HD, int G>
+template <int HD, int G, bool W8>
 static int launch_pair(const AttnItems& a, const Proj& p, int M, u16* y, int64_t ldy, int B, hipStream_t s) {
   const int Hq = a.Hkv * G;
   const size_t lds_att = (size_t)attn_item_lds_floats<HD, G>(a.chunk_max) * sizeof(float);
-  const size_t lds_band = stream_band_lds_bytes<PAIR_MT, PAIR_UNITS>();
+  const size_t lds_band = stream_band_lds_bytes<PAIR_MT, PAIR_UNITS, W8>();
   const size_t lds = lds_att > lds_band ? lds_att : lds_band;
   if (lds > 64 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_attn_beside_band<HD, G>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_attn_beside_band<HD, G, W8>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return LR_E_LAUNCH;
   }
-  k_attn_beside_band<HD, G><<<dim3((unsigned)(a.n_items + p.nwg)), dim3(256), lds, s>>>(a, p, M);
+  k_attn_beside_band<HD, G, W8><<<dim3((unsigned)(a.n_items + p.nwg)), dim3(256), lds, s>>>(a, p, M);
   k_attn_decode_combine<HD><<<dim3(Hq, B), dim3(HD), 0, s>>>(a.o_part, a.ml_part, y, ldy, Hq, a.nsplit);
   return lr_launch_status();
 }
 
-}  // namespace
-
-extern "C" int lr_attn_decode_beside(const void* q, int64_t ldq, const void* k_cache, const void* v_cache,
-                                     const int32_t* pos, void* y, int64_t ldy, int B, int Hq, int Hkv, int hd,
-                                     int Smax, void* scratch, size_t scratch_bytes, const lr_projection_t* proj,
-                                     int M, lr_stream_t stream) {
+// shared body of the two entry points; `fill` turns the caller's projection into a Proj
+template <bool W8, class Projection, class Fill>
+static int beside(const void* q, int64_t ldq, const void* k_cache, const void* v_cache, const int32_t* pos, void* y,
+                  int64_t ldy, int B, int Hq, int Hkv, int hd, int Smax, void* scratch, size_t scratch_bytes,
+                  const Projection* proj, int M, int m_min, lr_stream_t stream, Fill fill) {
   LR_REQUIRE_PTR(q);
   LR_REQUIRE_PTR(k_cache);
   LR_REQUIRE_PTR(v_cache);
@@ -80,9 +82,9 @@ extern "C" int lr_attn_decode_beside(const void* q, int64_t ldq, const void* k_c
   if (ldq % 8 || ldy % 8) return LR_E_ALIGN;
   if (scratch_bytes < lr_attn_decode_scratch_bytes(B, Hq, hd, Smax)) return LR_E_SHAPE;
   // the projection must not touch the cache the attention reads, and only the 16-row band shares a CU
-  if (proj->epilogue == LR_EPI_ROPE_KV || M > PAIR_MT) return LR_E_UNSUPPORTED;
+  if (proj->epilogue == LR_EPI_ROPE_KV || M > PAIR_MT || M < m_min) return LR_E_UNSUPPORTED;
   Proj p;
-  const int rc = sb_fill_projection(*proj, p);
+  const int rc = fill(*proj, p);
   if (rc != LR_OK) return rc;
   int G = Hq / Hkv;
   AttnItems a;
@@ -107,9 +109,28 @@ extern "C" int lr_attn_decode_beside(const void* q, int64_t ldq, const void* k_c
   plan(p, M, p.pair_off ? 16 : 16 * PAIR_UNITS, ncu);
   hipStream_t s = (hipStream_t)stream;
 #define LR_PAIR(HDV, GV) \
-  if (hd == HDV && G == GV) return launch_pair<HDV, GV>(a, p, M, (u16*)y, ldy, B, s);
+  if (hd == HDV && G == GV) return launch_pair<HDV, GV, W8>(a, p, M, (u16*)y, ldy, B, s);
   LR_PAIR(128, 1) LR_PAIR(128, 2) LR_PAIR(128, 4) LR_PAIR(128, 8)
   LR_PAIR(64, 1) LR_PAIR(64, 2) LR_PAIR(64, 4) LR_PAIR(64, 8)
 #undef LR_PAIR
   return LR_E_UNSUPPORTED;
+}
+
+}  // namespace
+
+extern "C" int lr_attn_decode_beside(const void* q, int64_t ldq, const void* k_cache, const void* v_cache,
+                                     const int32_t* pos, void* y, int64_t ldy, int B, int Hq, int Hkv, int hd,
+                                     int Smax, void* scratch, size_t scratch_bytes, const lr_projection_t* proj,
+                                     int M, lr_stream_t stream) {
+  return beside<false>(q, ldq, k_cache, v_cache, pos, y, ldy, B, Hq, Hkv, hd, Smax, scratch, scratch_bytes, proj, M, 1,
+                       stream, sb_fill_projection);
+}
+
+// (for one row lr_linear_fp8_multi uses the matrix-vector kernel, which has no band to put beside the attention)
+extern "C" int lr_attn_decode_beside_fp8(const void* q, int64_t ldq, const void* k_cache, const void* v_cache,
+                                         const int32_t* pos, void* y, int64_t ldy, int B, int Hq, int Hkv, int hd,
+                                         int Smax, void* scratch, size_t scratch_bytes,
+                                         const lr_projection_fp8_t* proj, int M, lr_stream_t stream) {
+  return beside<true>(q, ldq, k_cache, v_cache, pos, y, ldy, B, Hq, Hkv, hd, Smax, scratch, scratch_bytes, proj, M, LR_FP8_GEMV_MAX_M + 1,
+                      stream, sb_fill_projection_fp8);
 }

@@ -363,10 +363,16 @@ extern "C" int lr_linear_fp8(const void* x, int64_t ldx, const void* w8, const v
   return lr_launch_status();
 }
 
+namespace lr_detail {
+int stream_fp8_multi(const lr_projection_fp8_t* proj, int n_proj, int M, lr_stream_t stream);  // stream_gemm.hip
+}
+
 extern "C" int lr_linear_fp8_multi(const lr_projection_fp8_t* proj, int n_proj, int M, lr_stream_t stream) {
   if (proj == nullptr) return LR_E_NULL;
   if (n_proj < 1 || n_proj > 2 || M < 1) return LR_E_SHAPE;
-  if (M > 8) return LR_E_UNSUPPORTED;
+  if (M > 16) return LR_E_UNSUPPORTED;
+  // from 2 rows on the matrix cores: the dot products of the matrix-vector kernel grow with every row
+  if (M > LR_FP8_GEMV_MAX_M) return lr_detail::stream_fp8_multi(proj, n_proj, M, stream);
   P8 pr[2] = {};
   for (int i = 0; i < n_proj; ++i) {
     const int rc = fill_p8(proj[i], pr[i]);

@@ -9,6 +9,11 @@
 
 #define LR_WAVE 64
 
+// Weight-only e4m3 projections of a decode step (lr_linear_fp8_multi, lr_attn_decode_beside_fp8): up to this many
+// input rows the matrix-vector kernel, above it the matrix-core bands.  Measured on the 70B rank shard, ms per
+// step, kernel / bands: 1 row 3.66 / 3.77, 2 rows 4.40 / 3.77, 4 rows 5.22 / 3.96, 8 rows 8.13 / 4.19.
+constexpr int LR_FP8_GEMV_MAX_M = 1;
+
 typedef uint16_t u16;
 typedef uint32_t u32;
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));

@@ -27,6 +27,7 @@ struct Proj {
   int rpw;       // rows (row pairs if pair_off) per workgroup
   int pair_off;  // 0, or the distance from an up row to its gate row (= outputs)
   int nwg;       // workgroups of this projection
+  const u16* scales;  // weight-only e4m3 weights (the W8 kernels): one bf16 scale per weight row; else nullptr
   // RoPE + KV-cache epilogue of a fused q/k/v projection (rope_table == nullptr: none)
   const u16* rope_table;
   const int32_t* pos;
@@ -35,21 +36,43 @@ struct Proj {
   int Hq, Hkv, hd, Smax, block_size;
 };
 
-template <int MT, int UNITS>
+// the low (HI == false) or high two e4m3 values of a dword as a packed bf16 pair (exact)
+template <bool HI>
+__device__ __forceinline__ u32 sb_fp8_pair(u32 v) {
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v, 1.0f, HI));
+}
+
+template <int MT, int UNITS, bool W8 = false>
 constexpr size_t stream_band_lds_bytes() {
-  return (size_t)NWV * (UNITS * 16 * LROW + (MT >= LR_SG_XLDS_MIN ? MT * LROW : 0)) * sizeof(u16);
+  constexpr int LRW = (W8 ? 2 * KC : KC) + 8;
+  return (size_t)NWV * (UNITS * 16 * LRW + (MT >= LR_SG_XLDS_MIN ? MT * LRW : 0)) * sizeof(u16);
 }
 
 // One band of one projection, by the 256 lanes of a workgroup.  `sg_smem`: stream_band_lds_bytes<MT, UNITS>() bytes of LDS.
-template <int MT, int UNITS>
+// W8: the weights are e4m3 bytes with one bf16 scale per row (p.scales): a load instruction still covers 4 rows x
+// 256 bytes, now 256 elements of K, which are expanded to bf16 (exactly: e4m3 is a subset of bf16) on their way
+// into the LDS piece; the sum is rounded to bf16, multiplied by the row's scale and rounded again, as
+// F.linear(x, w.to(bf16)) * scales does, before the epilogue sees it.
+template <int MT, int UNITS, bool W8 = false>
 __device__ __forceinline__ void stream_band(const Proj& p, const int M, const int band, u16* sg_smem) {
-  constexpr int MTILES = MT / 16, KS = KC / 32, NLD = UNITS * 4;
+  static_assert(!W8 || MT == 16, "the e4m3 path is built for up to 16 input rows");
+  constexpr int KCW = W8 ? 256 : 128;  // k elements per chunk
+  constexpr int LRW = KCW + 8;         // LDS row length in elements
+  constexpr int WB = W8 ? 1 : 2;       // bytes per weight
+#ifndef LR_SG_W8_SETS
+#define LR_SG_W8_SETS 2
+#endif
+  // weight chunks in flight per wave: the e4m3 variant has twice the A fragments and input registers per chunk
+  // and gives up two of its four sets for a second workgroup per CU
+  constexpr int NS = W8 ? LR_SG_W8_SETS : SETS;
+  constexpr int MTILES = MT / 16, KS = KCW / 32, NLD = UNITS * 4;
   constexpr int NV = UNITS * MTILES * 4;  // accumulator registers per lane
   // From 32 input rows on the inputs too are loaded in whole lines (4 rows x 256 bytes per instruction) and take
   // the trip through LDS into B-fragment layout: L2 serves whole-line reads 1.5 times as fast as the 16 rows x
   // 64 bytes a fragment-layout load touches, and at 64 rows the input bytes are twice the weight bytes.
   constexpr bool XLDS = MT >= LR_SG_XLDS_MIN;
-  constexpr int WPIECE = UNITS * 16 * LROW, XPIECE = XLDS ? MT * LROW : 0;  // elements per wave
+  constexpr int WPIECE = UNITS * 16 * LRW, XPIECE = XLDS ? MT * LRW : 0;  // elements per wave
   // sg_smem: [NWV][WPIECE + XPIECE]
   static_assert(sizeof(float) * NV * 64 <= sizeof(u16) * WPIECE, "the partial sums reuse the wave's weight piece");
 
@@ -71,7 +94,9 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
   // ---- lane constants of the weight loads: instruction i covers band rows 4 i .. 4 i + 3 (in pair mode
   //      unit 0 holds the up rows, unit 1 the gate rows of the same pairs)
   const __amdgpu_buffer_rsrc_t wres =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<u16*>(wg_ + (int64_t)n0 * K), 0, 0x7fffffff, 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<unsigned char*>(reinterpret_cast<const unsigned char*>(wg_) + (int64_t)n0 * K * WB), 0, 0x7fffffff,
+          0x00020000);
   const __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc(const_cast<u16*>(xg), 0, 0x7fffffff, 0x00020000);
   int woff[NLD];
 #pragma unroll
@@ -79,7 +104,7 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
     const int r = 4 * i + l4;  // row inside the LDS piece
     int rr = r, extra = 0;
     if (pair_off && r >= 16) { rr = r - 16; extra = pair_off; }
-    woff[i] = rr < nrows ? (int)(((int64_t)(extra + rr) * K + l16 * 8) * 2) : OOB;
+    woff[i] = rr < nrows ? (int)((int64_t)(extra + rr) * K * WB + l16 * 16) : OOB;
   }
   // fragment layout: tile mt, k-step ks <- input row 16 mt + lane % 16, elements 32 ks + 8 (lane / 16) ..;
   // whole-line layout: instruction i <- input rows 4 i + lane / 16, elements 8 (lane % 16) ..
@@ -100,7 +125,7 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
   u16* const my = sg_smem + wave * (WPIECE + XPIECE);
   u16* const myx = my + WPIECE;
 
-  u32x4_t wr[SETS][NLD];
+  u32x4_t wr[NS][NLD];
   u32x4_t xr[2][MTILES][KS];
   f32x4_t acc[UNITS][MTILES];
 #pragma unroll
@@ -108,17 +133,17 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
 #pragma unroll
     for (int mt = 0; mt < MTILES; ++mt) acc[u][mt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-  // chunk ci of this wave starts at k0 = (ci * NWV + wave) * KC; what lies beyond K reads as zero (no
+  // chunk ci of this wave starts at k0 = (ci * NWV + wave) * KCW; what lies beyond K reads as zero (no
   // branch around a load: the number of loads in flight is fixed, so the waits between chunks are exact)
   auto issue_w = [&](int ci, u32x4_t (&dst)[NLD]) {
-    const int k0 = (ci * NWV + wave) * KC;
-    const bool kok = k0 + l16 * 8 < K;
+    const int k0 = (ci * NWV + wave) * KCW;
+    const bool kok = k0 + l16 * (16 / WB) < K;
 #pragma unroll
     for (int i = 0; i < NLD; ++i)
-      dst[i] = __builtin_amdgcn_raw_buffer_load_b128(wres, (kok && woff[i] != OOB) ? woff[i] : OOB, k0 * 2, LR_SG_W_AUX);
+      dst[i] = __builtin_amdgcn_raw_buffer_load_b128(wres, (kok && woff[i] != OOB) ? woff[i] : OOB, k0 * WB, LR_SG_W_AUX);
   };
   auto issue_x = [&](int ci, u32x4_t (&dst)[MTILES][KS]) {
-    const int k0 = (ci * NWV + wave) * KC;
+    const int k0 = (ci * NWV + wave) * KCW;
     if (XLDS) {
       const bool kok = k0 + l16 * 8 < K;
 #pragma unroll
@@ -137,34 +162,70 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
     }
   };
 
-  const int nck = (K + KC - 1) / KC;
+  const int nck = (K + KCW - 1) / KCW;
   const int nch = wave < nck ? (nck - wave + NWV - 1) / NWV : 0;  // chunks of this wave
   issue_x(0, xr[0]);
 #pragma unroll
-  for (int s = 0; s < SETS; ++s) issue_w(s, wr[s]);
-  for (int c0 = 0; c0 < nch; c0 += SETS) {
+  for (int s = 0; s < NS; ++s) issue_w(s, wr[s]);
+  for (int c0 = 0; c0 < nch; c0 += NS) {
 #pragma unroll
-    for (int s = 0; s < SETS; ++s) {
+    for (int s = 0; s < NS; ++s) {
       const int ci = c0 + s;
       issue_x(ci + 1, xr[(s + 1) & 1]);
       // ---- this chunk's weights: registers -> LDS (row-major) -> A fragments
       asm volatile("" ::: "memory");
 #pragma unroll
-      for (int i = 0; i < NLD; ++i)
-        *reinterpret_cast<u32x4_t*>(my + (4 * i + l4) * LROW + l16 * 8) = wr[s][i];
+      for (int i = 0; i < NLD; ++i) {
+        if constexpr (W8) {
+          u32x4_t lo, hi;
+          lo[0] = sb_fp8_pair<false>(wr[s][i][0]); lo[1] = sb_fp8_pair<true>(wr[s][i][0]);
+          lo[2] = sb_fp8_pair<false>(wr[s][i][1]); lo[3] = sb_fp8_pair<true>(wr[s][i][1]);
+          hi[0] = sb_fp8_pair<false>(wr[s][i][2]); hi[1] = sb_fp8_pair<true>(wr[s][i][2]);
+          hi[2] = sb_fp8_pair<false>(wr[s][i][3]); hi[3] = sb_fp8_pair<true>(wr[s][i][3]);
+          *reinterpret_cast<u32x4_t*>(my + (4 * i + l4) * LRW + l16 * 16) = lo;
+          *reinterpret_cast<u32x4_t*>(my + (4 * i + l4) * LRW + l16 * 16 + 8) = hi;
+        } else {
+          *reinterpret_cast<u32x4_t*>(my + (4 * i + l4) * LRW + l16 * 8) = wr[s][i];
+        }
+      }
       asm volatile("" ::: "memory");
+      if constexpr (W8) {
+        // 256 elements of K per chunk: the A fragments are taken in two halves to keep them at 32 registers
+        issue_w(ci + NS, wr[s]);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          bf16x8_t ah[UNITS][KS / 2];
+#pragma unroll
+          for (int u = 0; u < UNITS; ++u)
+#pragma unroll
+            for (int k2 = 0; k2 < KS / 2; ++k2)
+              ah[u][k2] =
+                  *reinterpret_cast<const bf16x8_t*>(my + (16 * u + l16) * LRW + (h * (KS / 2) + k2) * 32 + l4 * 8);
+#pragma unroll
+          for (int k2 = 0; k2 < KS / 2; ++k2)
+#pragma unroll
+            for (int mt = 0; mt < MTILES; ++mt) {
+              const bf16x8_t bx = __builtin_bit_cast(bf16x8_t, xr[s & 1][mt][h * (KS / 2) + k2]);
+#pragma unroll
+              for (int u = 0; u < UNITS; ++u)
+                acc[u][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah[u][k2], bx, acc[u][mt], 0, 0, 0);
+            }
+        }
+        asm volatile("" ::: "memory");
+        continue;
+      }
       bf16x8_t af[UNITS][KS];
 #pragma unroll
       for (int u = 0; u < UNITS; ++u)
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
-          af[u][ks] = *reinterpret_cast<const bf16x8_t*>(my + (16 * u + l16) * LROW + ks * 32 + l4 * 8);
+          af[u][ks] = *reinterpret_cast<const bf16x8_t*>(my + (16 * u + l16) * LRW + ks * 32 + l4 * 8);
       asm volatile("" ::: "memory");
-      issue_w(ci + SETS, wr[s]);
+      issue_w(ci + NS, wr[s]);
       if (XLDS) {
 #pragma unroll
         for (int i = 0; i < MT / 4; ++i)
-          *reinterpret_cast<u32x4_t*>(myx + (4 * i + l4) * LROW + l16 * 8) = xr[s & 1][i / KS][i % KS];
+          *reinterpret_cast<u32x4_t*>(myx + (4 * i + l4) * LRW + l16 * 8) = xr[s & 1][i / KS][i % KS];
         asm volatile("" ::: "memory");
       }
 #pragma unroll
@@ -172,7 +233,7 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
 #pragma unroll
         for (int mt = 0; mt < MTILES; ++mt) {
           bf16x8_t bx;
-          if (XLDS) bx = *reinterpret_cast<const bf16x8_t*>(myx + (16 * mt + l16) * LROW + ks * 32 + l4 * 8);
+          if (XLDS) bx = *reinterpret_cast<const bf16x8_t*>(myx + (16 * mt + l16) * LRW + ks * 32 + l4 * 8);
           else bx = __builtin_bit_cast(bf16x8_t, xr[s & 1][mt][ks]);
 #pragma unroll
           for (int u = 0; u < UNITS; ++u)
@@ -214,8 +275,12 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
         s0 += red[wv * WSTRIDE + ((u * MTILES + mt) * 4 + e) * 64 + ln];
         s1 += red[wv * WSTRIDE + ((u * MTILES + mt) * 4 + e + 1) * 64 + ln];
       }
-      const float x0 = round_bf(s0), x1 = round_bf(s1);
       const int n = n0 + r;
+      float x0 = round_bf(s0), x1 = round_bf(s1);
+      if constexpr (W8) {
+        x0 = round_bf(x0 * bf_to_f(pp.scales[n]));
+        x1 = round_bf(x1 * bf_to_f(pp.scales[n + 1]));
+      }
       u32 plain = pack_bf2(x0, x1), out = plain;
       if (in_range) {
         const int sect = n < nq ? 0 : (n < nq + nkv ? 1 : 2);
@@ -248,7 +313,14 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
 #pragma unroll
         for (int wv = 0; wv < NWV; ++wv) s1 += red[wv * WSTRIDE + ((MTILES + mt) * 4 + e) * 64 + ln];
       }
-      yg[(int64_t)m * ldy + n0 + r] = f_to_bf(swiglu_bf(round_bf(s0), round_bf(s1)));
+      float u_ = round_bf(s0), g_ = round_bf(s1);
+      if constexpr (W8) {
+        u_ = round_bf(u_ * bf_to_f(p.scales[n0 + r]));
+        g_ = round_bf(g_ * bf_to_f(p.scales[pair_off + n0 + r]));
+      }
+      yg[(int64_t)m * ldy + n0 + r] = f_to_bf(swiglu_bf(u_, g_));
+    } else if constexpr (W8) {
+      yg[(int64_t)m * ldy + n0 + r] = f_to_bf(round_bf(s0) * bf_to_f(p.scales[n0 + r]));
     } else {
       yg[(int64_t)m * ldy + n0 + r] = f_to_bf(s0);
     }
@@ -314,6 +386,20 @@ static int sb_fill_projection(const lr_projection_t& q, Proj& p) {
     p.err = r->err; p.Hq = r->n_head; p.Hkv = r->n_kv_head; p.hd = r->head_dim; p.Smax = r->smax;
     p.block_size = r->block_size;
   }
+  return LR_OK;
+}
+
+// lr_projection_fp8_t -> Proj for the e4m3 bands (W8 = true)
+static int sb_fill_projection_fp8(const lr_projection_fp8_t& q, Proj& p) {
+  if (q.scales == nullptr) return LR_E_NULL;
+  if (lr_misaligned(q.w8)) return LR_E_ALIGN;
+  if (q.K % 16) return LR_E_ALIGN;
+  // the bf16 projection's checks, with the weight pointer standing in (its rows are half as long: every
+  // 32-bit offset limit holds a fortiori)
+  const lr_projection_t as_bf16 = {q.x, q.ldx, q.w8, q.y, q.ldy, q.N, q.K, q.epilogue, q.rope};
+  const int rc = sb_fill_projection(as_bf16, p);
+  if (rc != LR_OK) return rc;
+  p.scales = (const u16*)q.scales;
   return LR_OK;
 }
 

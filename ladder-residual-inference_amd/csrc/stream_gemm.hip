@@ -24,31 +24,43 @@
 
 namespace {
 
-template <int MT, int UNITS>
+template <int MT, int UNITS, bool W8>
 __global__ __launch_bounds__(NWV * 64) void k_stream_gemm(const Proj p0, const Proj p1, const int M) {
   extern __shared__ __attribute__((aligned(16))) u16 sg_smem[];
   const bool second = (int)blockIdx.x >= p0.nwg;
   const Proj p = second ? p1 : p0;
-  stream_band<MT, UNITS>(p, M, second ? (int)blockIdx.x - p0.nwg : (int)blockIdx.x, sg_smem);
+  stream_band<MT, UNITS, W8>(p, M, second ? (int)blockIdx.x - p0.nwg : (int)blockIdx.x, sg_smem);
 }
 
-template <int MT, int UNITS>
+template <int MT, int UNITS, bool W8 = false>
 static int launch_units(Proj& a, Proj& b, int M, hipStream_t s) {
-  constexpr size_t lds = stream_band_lds_bytes<MT, UNITS>();
+  constexpr size_t lds = stream_band_lds_bytes<MT, UNITS, W8>();
   static bool attr_set = false;
   if (!attr_set && lds > 64 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_stream_gemm<MT, UNITS>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_stream_gemm<MT, UNITS, W8>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return LR_E_LAUNCH;
     attr_set = true;
   }
-  k_stream_gemm<MT, UNITS><<<dim3((unsigned)(a.nwg + b.nwg)), dim3(NWV * 64), lds, s>>>(a, b, M);
+  k_stream_gemm<MT, UNITS, W8><<<dim3((unsigned)(a.nwg + b.nwg)), dim3(NWV * 64), lds, s>>>(a, b, M);
   return LR_OK;
 }
 
 template <int MT>
 static int launch(Proj& a, Proj& b, int M, int units, hipStream_t s) {
   return units == 2 ? launch_units<MT, 2>(a, b, M, s) : launch_units<MT, 1>(a, b, M, s);
+}
+
+// one 16-row unit per workgroup when every CU still gets a band that way; row pairs always take two units
+static int pick_units_and_plan(Proj* pr, int n_proj, int M, int ncu) {
+  bool any_pair = false, all_thin = true;
+  for (int i = 0; i < n_proj; ++i) {
+    any_pair = any_pair || pr[i].pair_off != 0;
+    if (pr[i].N > 16 * ncu) all_thin = false;
+  }
+  const int units = (any_pair || !all_thin) ? 2 : 1;
+  for (int i = 0; i < n_proj; ++i) plan(pr[i], M, pr[i].pair_off ? 16 : 16 * units, ncu);
+  return units;
 }
 
 }  // namespace
@@ -58,22 +70,33 @@ extern "C" int lr_linear_multi(const lr_projection_t* proj, int n_proj, int M, l
   if (n_proj < 1 || n_proj > 2 || M < 1) return LR_E_SHAPE;
   if (M > 64) return LR_E_UNSUPPORTED;
   Proj pr[2] = {};
-  bool any_pair = false;
   for (int i = 0; i < n_proj; ++i) {
     const int rc = sb_fill_projection(proj[i], pr[i]);
     if (rc != LR_OK) return rc;
-    any_pair = any_pair || pr[i].pair_off != 0;
   }
   const int ncu = sb_num_cus();
   if (ncu < 1) return LR_E_LAUNCH;
-  bool all_thin = true;
-  for (int i = 0; i < n_proj; ++i)
-    if (pr[i].N > 16 * ncu) all_thin = false;
-  // one 16-row unit per workgroup when every CU still gets a band that way; row pairs always take two units
-  const int units = (any_pair || !all_thin) ? 2 : 1;
-  for (int i = 0; i < n_proj; ++i) plan(pr[i], M, pr[i].pair_off ? 16 : 16 * units, ncu);
+  const int units = pick_units_and_plan(pr, n_proj, M, ncu);
   hipStream_t s = (hipStream_t)stream;
   const int rc = M <= 16 ? launch<16>(pr[0], pr[1], M, units, s)
                  : (M <= 32 ? launch<32>(pr[0], pr[1], M, units, s) : launch<64>(pr[0], pr[1], M, units, s));
   return rc != LR_OK ? rc : lr_launch_status();
 }
+
+// lr_linear_fp8_multi (gemv_fp8.hip) for 3 to 16 input rows: the same bands with e4m3 weights.
+namespace lr_detail {
+int stream_fp8_multi(const lr_projection_fp8_t* proj, int n_proj, int M, lr_stream_t stream) {
+  if (M < 1 || M > 16) return LR_E_UNSUPPORTED;
+  Proj pr[2] = {};
+  for (int i = 0; i < n_proj; ++i) {
+    const int rc = sb_fill_projection_fp8(proj[i], pr[i]);
+    if (rc != LR_OK) return rc;
+  }
+  const int ncu = sb_num_cus();
+  if (ncu < 1) return LR_E_LAUNCH;
+  const int units = pick_units_and_plan(pr, n_proj, M, ncu);
+  hipStream_t s = (hipStream_t)stream;
+  const int rc = units == 2 ? launch_units<16, 2, true>(pr[0], pr[1], M, s) : launch_units<16, 1, true>(pr[0], pr[1], M, s);
+  return rc != LR_OK ? rc : lr_launch_status();
+}
+}  // namespace lr_detail

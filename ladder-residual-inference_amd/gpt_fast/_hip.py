@@ -40,6 +40,8 @@ _PROTOS = {
                                c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "lr_attn_decode_beside": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,
                                       c_int, c_int, c_int, c_void_p, c_size_t, c_void_p, c_int, c_void_p]),
+    "lr_attn_decode_beside_fp8": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int,
+                                          c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p, c_int, c_void_p]),
     "lr_attn_decode_static": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,
                                       c_int, c_int, c_int, c_void_p]),
     "lr_attn_prefill": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,
@@ -251,8 +253,30 @@ class _ProjectionFp8(ctypes.Structure):
 
 
 def linear_fp8_multi(*projections):
-    """linear_multi for weight-only e4m3 projections of the same M <= 8 rows (lr_linear_fp8_multi).  Each projection
+    """linear_multi for weight-only e4m3 projections of the same M <= 16 rows (lr_linear_fp8_multi).  Each projection
     is (x [M, K], w8 [N, K] float8_e4m3fn, scales [N], out, epilogue), epilogue as in linear_multi."""
+    arr, M, _keep = _projection_fp8_array(projections)
+    _check(load().lr_linear_fp8_multi(ctypes.cast(arr, c_void_p), len(projections), M, _stream()), "lr_linear_fp8_multi")
+
+
+def attn_decode_beside_fp8(q, k_cache, v_cache, pos, y, scratch, B, Hq, Hkv, hd, projection) -> bool:
+    """attn_decode and linear_fp8_multi(projection) in one launch (lr_attn_decode_beside_fp8); False, with nothing
+    launched, when the library has no such kernel for the shape (a single row among them)."""
+    _, _, ldq = _rows_ld(q)
+    _, _, ldy = _rows_ld(y)
+    Smax = k_cache.shape[2]
+    assert pos.dtype == torch.int32 and pos.numel() == 1 and scratch.dtype == torch.float32
+    arr, M, _keep = _projection_fp8_array((projection,))
+    rc = load().lr_attn_decode_beside_fp8(_dev(q), ldq, _dev(k_cache), _dev(v_cache), pos.data_ptr(), _dev(y), ldy, B,
+                                          Hq, Hkv, hd, Smax, scratch.data_ptr(), scratch.numel() * 4,
+                                          ctypes.cast(arr, c_void_p), M, _stream())
+    if rc == E_UNSUPPORTED:
+        return False
+    _check(rc, "lr_attn_decode_beside_fp8")
+    return True
+
+
+def _projection_fp8_array(projections):
     arr = (_ProjectionFp8 * len(projections))()
     M = None
     keep = []
@@ -271,7 +295,7 @@ def linear_fp8_multi(*projections):
         M = m
         arr[i] = _ProjectionFp8(_dev(x), ldx, w8.data_ptr(), _dev(scales), _dev(out), ldy, N, K, epi,
                                 ctypes.pointer(rope) if rope is not None else None)
-    _check(load().lr_linear_fp8_multi(ctypes.cast(arr, c_void_p), len(projections), M, _stream()), "lr_linear_fp8_multi")
+    return arr, M, keep
 
 
 def linear_fp8(x: torch.Tensor, w8: torch.Tensor, scales: torch.Tensor, out: torch.Tensor):

@@ -144,8 +144,9 @@ class GPTLadder(GPTBase):
         fp8 = hasattr(self.layers[0].attention.wqkv, "scales")
         multi = side is None and ws.B <= 64 and not fp8
         beside = multi and ws.B <= 16
-        # weight-only e4m3 projections, up to 8 rows: the same two launches per block from the fp8 matrix-vector kernel
-        multi8 = side is None and fp8 and ws.B <= 8
+        # weight-only e4m3 projections, up to 16 rows: the same two launches per block (lr_linear_fp8_multi)
+        multi8 = side is None and fp8 and ws.B <= 16
+        beside8 = multi8   # (declined by the library for a single row, where the projections are no bands)
         for blk in self.layers:
             _hip.ladder_norms(ws.x, pending_a, pending_m, blk.attention_norm.weight, blk.ffn_norm.weight, ws.x, ws.xn,
                               ws.xn2, eps)
@@ -172,9 +173,18 @@ class GPTLadder(GPTBase):
                 att, ff, kv = blk.attention, blk.feed_forward, blk.attention.kv_cache
                 rope = _hip.rope_kv_epilogue(self.freqs_cis, pos, kv.k_cache, kv.v_cache, cfg.n_head_local,
                                              cfg.n_kv_local, cfg.head_dim)
-                _hip.linear_fp8_multi((ws.xn, att.wqkv.weight, att.wqkv.scales, ws.qkv, rope),
-                                      (ws.xn2, ff.w1.weight, ff.w1.scales, ws.act, _hip.EPI_SWIGLU))
-                self._attention(ws, blk, pos, None, None, roped=True)
+                qkv8 = (ws.xn, att.wqkv.weight, att.wqkv.scales, ws.qkv, rope)
+                up_gate8 = (ws.xn2, ff.w1.weight, ff.w1.scales, ws.act, _hip.EPI_SWIGLU)
+                if beside8:
+                    _hip.linear_fp8_multi(qkv8)
+                    beside8 = _hip.attn_decode_beside_fp8(ws.qkv, kv.k_cache, kv.v_cache, pos, ws.y, ws.scratch, ws.B,
+                                                          cfg.n_head_local, cfg.n_kv_local, cfg.head_dim, up_gate8)
+                    if not beside8:
+                        _hip.linear_fp8_multi(up_gate8)
+                        self._attention(ws, blk, pos, None, None, roped=True)
+                else:
+                    _hip.linear_fp8_multi(qkv8, up_gate8)
+                    self._attention(ws, blk, pos, None, None, roped=True)
                 _hip.linear_fp8_multi((ws.y, att.wo.weight, att.wo.scales, ws.a, _hip.EPI_NONE),
                                       (ws.act, ff.w2.weight, ff.w2.scales, ws.m, _hip.EPI_NONE))
             elif side is not None:

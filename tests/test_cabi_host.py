@@ -93,7 +93,7 @@ def test_validation_precedes_any_device_work(lib):
     one8 = (_ProjectionFp8 * 1)(_ProjectionFp8(64, 16, 128, 192, 256, 8, 8, 16, 0))
     ptr8 = ctypes.cast(one8, ctypes.c_void_p)
     assert lib.lr_linear_fp8_multi(None, 1, 1, None) == E_NULL
-    assert lib.lr_linear_fp8_multi(ptr8, 1, 9, None) == -4            # the matrix-vector kernel takes up to 8 rows
+    assert lib.lr_linear_fp8_multi(ptr8, 1, 17, None) == -4           # up to 16 rows
     assert lib.lr_linear_fp8_multi(ptr8, 3, 1, None) == E_SHAPE
     one8[0].K = 24                                                    # 16 weights per lane and load
     assert lib.lr_linear_fp8_multi(ptr8, 1, 1, None) == E_SHAPE       # ldx < K
