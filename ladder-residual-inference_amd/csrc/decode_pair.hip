@@ -131,6 +131,6 @@ extern "C" int lr_attn_decode_beside_fp8(const void* q, int64_t ldq, const void*
                                          const int32_t* pos, void* y, int64_t ldy, int B, int Hq, int Hkv, int hd,
                                          int Smax, void* scratch, size_t scratch_bytes,
                                          const lr_projection_fp8_t* proj, int M, lr_stream_t stream) {
-  return beside<true>(q, ldq, k_cache, v_cache, pos, y, ldy, B, Hq, Hkv, hd, Smax, scratch, scratch_bytes, proj, M, LR_FP8_GEMV_MAX_M + 1,
-                      stream, sb_fill_projection_fp8);
+  return beside<true>(q, ldq, k_cache, v_cache, pos, y, ldy, B, Hq, Hkv, hd, Smax, scratch, scratch_bytes, proj, M,
+                      LR_FP8_GEMV_MAX_M + 1, stream, sb_fill_projection_fp8);
 }
