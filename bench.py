@@ -219,6 +219,8 @@ def main():
     ap.add_argument("--per-op", action="store_true",
                     help="decode with one kernel per operation (captured in the hipGraph) instead of the persistent "
                          "one-kernel step: the comparison point, not the headline")
+    ap.add_argument("--fp8", action="store_true",
+                    help="weight-only e4m3 projections (gpt_fast.quantize): a profiling aid, not the headline")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (reads 1 GiB, writes 1 GiB) a few times: under "
                          "rocprofv3 --pmc its FETCH_SIZE / WRITE_SIZE readings calibrate the counters' unit")
@@ -241,6 +243,10 @@ def main():
     model.last_logits_only = True          # prefill is set-up here, not the timed region
     if args.per_op:
         model.use_fused_step = False
+    if args.fp8:
+        from gpt_fast.quantize import quantize_model_fp8
+
+        quantize_model_fp8(model)
     cfg = model.config
     new = max(K, W, 127) + 1
     g = torch.Generator(device=dev)
@@ -280,13 +286,14 @@ def main():
     ms_per_step = 1e3 * elapsed / K
     tokens = dg.history[0, : min(K, 16)].tolist()
 
-    step_bytes = sum(bm.decode_bytes_per_step(cfg, B, T + i) for i in range(K)) / K
+    bytes_per_step = fp8_bytes_per_step if args.fp8 else bm.decode_bytes_per_step
+    step_bytes = sum(bytes_per_step(cfg, B, T + i) for i in range(K)) / K
     step_gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
 
     # ---- dominant kernel, timed with HIP events on the stream it is launched on (torch's current stream)
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     fused = getattr(model, "use_fused_step", False) and hasattr(model, "decode_step_fused") and \
-        model._fused_step(B) is not None
+        model._fused_step(B) is not None and not args.fp8
     if fused:
         # the whole step is ONE kernel (k_ladder_step): algorithmic bytes per launch = bytes per step
         pos = torch.tensor([T], dtype=torch.int32, device=dev)
@@ -312,19 +319,29 @@ def main():
         N, Kdim = w1s[0].shape
         x = torch.randn(B, Kdim, device=dev).to(torch.bfloat16)
         y = torch.empty(B, N, device=dev, dtype=torch.bfloat16)
-        for w in w1s[:8]:
-            _hip.linear(x, w, y)
+        if args.fp8:
+            scs = [(blk.feed_forward.w1 if hasattr(blk, "feed_forward") else blk.attention.wqkv1).scales
+                   for blk in model.layers]
+            run = lambda i: _hip.linear_fp8_multi((x, w1s[i], scs[i], y, _hip.EPI_NONE)) if B <= 16 else \
+                _hip.linear_fp8(x, w1s[i], scs[i], y)
+        else:
+            run = lambda i: _hip.linear(x, w1s[i], y)
+        for i in range(8):
+            run(i)
         reps = 3
         torch.cuda.synchronize()
         ev0.record()
         for _ in range(reps):
-            for w in w1s:
-                _hip.linear(x, w, y)
+            for i in range(len(w1s)):
+                run(i)
         ev1.record()
         torch.cuda.synchronize()
         k_us = 1e3 * ev0.elapsed_time(ev1) / (reps * len(w1s))
-        k_bytes = 2 * (N * Kdim + B * Kdim + B * N)
-        k_name = f"k_gemv (w1 up+gate projection, [{N} x {Kdim}] bf16, M={B})"
+        wbytes = 1 if args.fp8 else 2
+        k_bytes = wbytes * N * Kdim + 2 * (B * Kdim + B * N)
+        kern = ("k_gemv_fp8_multi" if B == 1 else "k_stream_gemm (e4m3 bands)") if args.fp8 else \
+            ("k_gemv" if B <= 4 else "k_stream_gemm")
+        k_name = f"{kern} (w1 up+gate projection, [{N} x {Kdim}] {'e4m3' if args.fp8 else 'bf16'}, M={B})"
     k_gbps = k_bytes / (k_us * 1e-6) / 1e9
 
     # ---- the read rate this machine reaches: a plain streaming read of 8 GiB by every CU
@@ -345,11 +362,13 @@ def main():
     out = {
         "metric": "decode_tokens_per_sec", "value": round(B * 1e3 / ms_per_step, 2), "unit": "tok/s",
         "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16 (e4m3 weights)" if args.fp8 else "bf16",
+        "data": "synthetic",
         "config": {"workload": f"{args.model} rank shard (dim {cfg.dim}, {cfg.n_layer} layers, {cfg.n_head_local} q / "
                                f"{cfg.n_kv_local} kv heads, FFN {cfg.ffn_local}, lm_head rows {cfg.output_rows}), "
                                f"batch {B}, prompt {T}, greedy decode, hipGraph replay per step"
-                               + (", one kernel per operation" if args.per_op else ""),
+                               + (", one kernel per operation" if args.per_op else "")
+                               + (", weight-only e4m3 projections" if args.fp8 else ""),
                    "batch": B, "prompt_len": T, "virtual_tp": cfg.tp_world_size},
         "ms_per_token": round(ms_per_step, 4),
         "prefill_s": round(prefill_s, 4),

@@ -172,10 +172,11 @@ int lr_attn_decode_beside(const void* q, int64_t ldq, const void* k_cache, const
  * holding `weight` in the narrow type and `scales` in the model dtype (gpt_ladder_TP.py:233-237) --
  * whose forward is F.linear(x, weight.to(x.dtype)) * scales; this is that forward with e4m3 weights
  * (the reference ships no quantiser and no quantised layer, so parity at this boundary is pinned by
- * the formula only).  M <= 8 (decode) streams the fp8 weights once: half the HBM bytes of lr_linear.
- * M > 8 (prefill) expands the weights to bf16 into `scratch` (lr_linear_fp8_scratch_bytes(M, N, K)
+ * the formula only).  M <= 16 (decode) streams the fp8 weights once: half the HBM bytes of lr_linear
+ * (one row: matrix-vector kernel; 2 to 16 rows: the matrix-core bands of lr_linear_fp8_multi).
+ * M > 16 (prefill) expands the weights to bf16 into `scratch` (lr_linear_fp8_scratch_bytes(M, N, K)
  * bytes, 16-byte aligned), runs lr_linear on them and scales the columns; scratch may be NULL for
- * M <= 8. */
+ * M <= 16. */
 size_t lr_linear_fp8_scratch_bytes(int M, int N, int K);
 int lr_linear_fp8(const void* x, int64_t ldx, const void* w8, const void* scales, void* y, int64_t ldy, int M, int N,
                   int K, void* scratch, size_t scratch_bytes, lr_stream_t stream);

@@ -7,8 +7,10 @@
 // rounded to bf16, multiplied by the row's scale and rounded again -- the two roundings of
 // F.linear(x, w.to(bf16)) * scales.  Partial sums meet in a fixed order: bit-reproducible.
 //
-// For more than 8 input rows (prefill) the weights are expanded to bf16 in a caller-provided scratch
-// buffer and the bf16 matrix-core GEMM runs on that, followed by the per-column scaling.
+// From 2 to 16 input rows (decode batches) the projections run as matrix-core bands that expand the
+// weights on their way through LDS (stream_band.h, W8).  For more than 16 input rows (prefill) the
+// weights are expanded to bf16 in a caller-provided scratch buffer and the bf16 matrix-core GEMM runs
+// on that, followed by the per-column scaling.
 #include "lr_common.h"
 
 namespace {
@@ -326,8 +328,12 @@ __global__ __launch_bounds__(256) void k_scale_cols(u16* __restrict__ y, int64_t
 
 }  // namespace
 
+namespace lr_detail {
+int stream_fp8_multi(const lr_projection_fp8_t* proj, int n_proj, int M, lr_stream_t stream);  // stream_gemm.hip
+}
+
 extern "C" size_t lr_linear_fp8_scratch_bytes(int M, int N, int K) {
-  if (M <= 8 || N <= 0 || K <= 0) return 0;
+  if (M <= 16 || N <= 0 || K <= 0) return 0;
   return (size_t)N * K * 2;
 }
 
@@ -344,6 +350,12 @@ extern "C" int lr_linear_fp8(const void* x, int64_t ldx, const void* w8, const v
   const unsigned char* wp = (const unsigned char*)w8;
   const u16* sp = (const u16*)scales;
   u16* yp = (u16*)y;
+  if (M > LR_FP8_GEMV_MAX_M && M <= 16 && !lr_misaligned(scales)) {
+    // decode batches: the matrix-core bands of lr_linear_fp8_multi (one projection, no epilogue)
+    const lr_projection_fp8_t one = {x, ldx, w8, scales, y, ldy, N, K, LR_EPI_NONE, nullptr};
+    const int rc = lr_detail::stream_fp8_multi(&one, 1, M, stream);
+    if (rc != LR_E_UNSUPPORTED || M > 8) return rc;
+  }
   if (M <= 8) {
     if (M == 1) launch<1>(xp, ldx, wp, sp, yp, ldy, M, N, K, s);
     else if (M == 2) launch<2>(xp, ldx, wp, sp, yp, ldy, M, N, K, s);
@@ -361,10 +373,6 @@ extern "C" int lr_linear_fp8(const void* x, int64_t ldx, const void* w8, const v
   if (M > 65535) return LR_E_UNSUPPORTED;
   k_scale_cols<<<dim3((N + 255) / 256 < 64 ? (N + 255) / 256 : 64, M), dim3(256), 0, s>>>(yp, ldy, sp, N);
   return lr_launch_status();
-}
-
-namespace lr_detail {
-int stream_fp8_multi(const lr_projection_fp8_t* proj, int n_proj, int M, lr_stream_t stream);  // stream_gemm.hip
 }
 
 extern "C" int lr_linear_fp8_multi(const lr_projection_fp8_t* proj, int n_proj, int M, lr_stream_t stream) {

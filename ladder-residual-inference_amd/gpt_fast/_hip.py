@@ -299,7 +299,7 @@ def _projection_fp8_array(projections):
 
 
 def linear_fp8(x: torch.Tensor, w8: torch.Tensor, scales: torch.Tensor, out: torch.Tensor):
-    """out[M, N] = (x[M, K] @ w8[N, K]^T rounded to bf16) * scales[N]: weight-only e4m3 linear.  For M > 8 the
+    """out[M, N] = (x[M, K] @ w8[N, K]^T rounded to bf16) * scales[N]: weight-only e4m3 linear.  For M > 16 the
     expanded weights go through a per-device scratch buffer that grows to the largest matrix seen (allocated
     here, outside the library; allocate it before capturing a graph by running the shape once)."""
     M, K, ldx = _rows_ld(x)

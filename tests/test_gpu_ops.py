@@ -412,10 +412,11 @@ def test_linear_fp8_decodes_every_e4m3_value_exactly(hip):
 
 @pytest.mark.parametrize("N,K", [(1280, 8192), (8192, 1024), (7168, 8192), (8192, 3584), (16032, 8192), (3072, 2048),
                                  (1001, 528), (24, 64)])
-@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 16, 300])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 16, 17, 300])
 def test_linear_fp8(hip, M, N, K):
-    """Decode (M <= 8: fp8 weights streamed once) and prefill (M > 8: expanded to bf16 in scratch + matrix-core
-    GEMM + column scaling) against the oracle's F.linear(x, w8.to(bf16)) * scales."""
+    """Decode (one row: matrix-vector kernel; 2 to 16 rows: matrix-core bands; fp8 weights streamed once) and prefill
+    (M > 16: expanded to bf16 in scratch + matrix-core GEMM + column scaling) against the oracle's
+    F.linear(x, w8.to(bf16)) * scales."""
     if M == 300 and N * K > 30e6:
         M = 64
     x = rnd(M, K, seed=40)
