@@ -1222,6 +1222,14 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
     const unsigned tag = tag_of(epoch_base + (unsigned)t + 1u), tag_prev = tag_of(epoch_base + (unsigned)t);
     const unsigned act_wo = p.oact + (unsigned)((t & 1) * M * I);  // activations alternate between two buffers
     LR_STAMP(1)
+#ifdef LR_STEP_PROFILE
+    // where this workgroup runs: XCC_ID (hardware register 20) above the low 16 bits of HW_ID (register 4: wave,
+    // SIMD, pipe, CU, shader array, shader engine), in stamp 9
+    if (p.prof && t >= p.prof_t0 && t < p.prof_t0 + PROF_SLOTS && tid == 0)
+      p.prof[((size_t)blockIdx.x * PROF_SLOTS + (t - p.prof_t0)) * PROF_POINTS + 9] =
+          ((unsigned long long)__builtin_amdgcn_s_getreg((31 << 11) | 20) << 16) |
+          (__builtin_amdgcn_s_getreg((15 << 11) | 4) & 0xffffu);
+#endif
     const Job j_qkv = LR_JOB(JK_QKV, LP_WQKV);
     // m(t-1) for the coming residual step: on its way while the query/key/value rows are done
     issue_words<M>(coh, t >= 1, p.om, D, ew);

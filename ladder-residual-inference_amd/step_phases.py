@@ -6,7 +6,8 @@
 The profile build of the step kernel writes, per workgroup, a 100 MHz wall-clock stamp at every phase boundary of
 four consecutive layer slots (lr_ladder_step_profile, profile builds only).  This script runs a few steps of the
 benchmark workload (random weights, batch 1) on that library and prints, per phase, the mean / min / max duration
-over the workgroups -- attention workgroups and weight-streaming workgroups separately -- and the slot length."""
+over the workgroups -- attention workgroups and weight-streaming workgroups separately -- the slot length, and
+which workgroups (on which XCD / shader engine / CU) finish the slot last."""
 import argparse
 import ctypes
 import os
@@ -88,6 +89,15 @@ def main():
     print("  slot length (loop top to loop top), three consecutive slots: " + ", ".join(f"{x:.2f}" for x in lens))
     ends = a[:, s, 8] - a[:, s, 1].min()
     print(f"  w2 finish time after the first workgroup entered the slot: mean {ends.mean():.2f}, last {ends.max():.2f}")
+    # stamp 9 holds where the workgroup runs: XCC_ID above the low 16 bits of HW_ID (CU [11:8], SH [12], SE [15:13])
+    hw = buf.cpu().numpy().reshape(-1, 4, 16)[:, s, 9]
+    xcc, se, cu = (hw >> 16) & 0xF, (hw >> 13) & 0x7, (hw >> 8) & 0xF
+    last = np.argsort(ends)[-6:][::-1]
+    print("  the six workgroups that finish w2 last (workgroup: XCD / shader engine / CU, lag behind the mean):")
+    print("    " + ", ".join(f"{w}: {xcc[w]}/{se[w]}/{cu[w]} +{ends[w] - ends.mean():.1f}" for w in last))
+    lag1 = a[last, s, 4] - a[:, s, 4].mean()
+    print("    the same six at the end of w1 | attention: " + ", ".join(f"+{x:.1f}" for x in lag1))
+    print("  mean w2 finish per XCD: " + ", ".join(f"{ends[xcc == x].mean():.1f}" for x in range(int(xcc.max()) + 1)))
 
 
 if __name__ == "__main__":
