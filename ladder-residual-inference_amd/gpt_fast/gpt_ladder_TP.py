@@ -120,6 +120,7 @@ class GPTLadder(GPTBase):
     # shard, ms per step with / without: batch 8 8.6 / 8.3, batch 64 18.2 / 18.8).  Putting one step of each chain
     # into the same grid instead (wqkv beside w1, attention beside w2) was slower still: 10.3 ms at batch 8.
     overlap_modules = False
+    two_chains_from = 33   # decode batches from which the MLP chain is a parallel branch (see _run_layers_decode)
 
     def _run_layers_decode(self, ws: Workspace, pos: Tensor):
         """Decode step (S == 1) of an all-ladder model through the per-op kernels: one launch does both residual
@@ -144,6 +145,16 @@ class GPTLadder(GPTBase):
         fp8 = hasattr(self.layers[0].attention.wqkv, "scales")
         multi = side is None and ws.B <= 64 and not fp8
         beside = multi and ws.B <= 16
+        # Above 32 rows a band workgroup fills the register file of its waves but not the CU: the MLP chain (up/gate,
+        # w2) runs as a second branch of the captured graph beside the attention chain (q/k/v, attention, wo) --
+        # 70B rank shard, batch 64: 10.4 -> 9.9 ms per step; at batch 32 nothing moves (7.35 / 7.31), below that
+        # the attention shares the up/gate launch instead
+        two_chains = multi and not beside and ws.B >= self.two_chains_from
+        if two_chains:
+            cur = torch.cuda.current_stream()
+            chain = getattr(self, "_chain_stream", None)
+            if chain is None or chain.device != cur.device:
+                chain = self._chain_stream = torch.cuda.Stream(device=cur.device)
         # weight-only e4m3 projections, up to 16 rows: the same two launches per block (lr_linear_fp8_multi)
         multi8 = side is None and fp8 and ws.B <= 16
         beside8 = multi8   # (declined by the library for a single row, where the projections are no bands)
@@ -164,6 +175,17 @@ class GPTLadder(GPTBase):
                     if not beside:
                         _hip.linear_multi(up_gate)
                         self._attention(ws, blk, pos, None, None, roped=True)
+                elif two_chains:
+                    chain.wait_stream(cur)
+                    with torch.cuda.stream(chain):
+                        _hip.linear_multi(up_gate)
+                        _hip.linear_multi((ws.act, blk.feed_forward.w2.weight, ws.m, _hip.EPI_NONE))
+                    _hip.linear_multi((ws.xn, blk.attention.wqkv.weight, ws.qkv, rope))
+                    self._attention(ws, blk, pos, None, None, roped=True)
+                    _hip.linear_multi((ws.y, blk.attention.wo.weight, ws.a, _hip.EPI_NONE))
+                    cur.wait_stream(chain)
+                    pending_a, pending_m = ws.a, ws.m
+                    continue
                 else:
                     _hip.linear_multi((ws.xn, blk.attention.wqkv.weight, ws.qkv, rope), up_gate)
                     self._attention(ws, blk, pos, None, None, roped=True)

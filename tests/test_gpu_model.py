@@ -191,6 +191,16 @@ def test_tiny_ladder_per_op_decode_modes(B, mode):
     check(stats)
 
 
+def test_tiny_ladder_mlp_chain_as_a_parallel_graph_branch():
+    """Above 16 sequences the MLP chain can run beside the attention chain as a second branch of the captured graph
+    (the default from 33 sequences on): same tokens and logits as the oracle, replays equal to eager."""
+    model = build("ladder", **dict(TINY, dim=512, n_head=8, n_local_heads=2, intermediate_size=640))
+    model.two_chains_from = 17
+    stats = run_parity(model, "ladder", B=20, T=20, new=12, fused=False)
+    print(stats)
+    check(stats)
+
+
 def test_tiny_ladder_fused_head_dim_128_many_kv_heads():
     kw = dict(TINY, block_size=128, n_head=8, n_local_heads=2, dim=1024, intermediate_size=768, n_layer=2,
               vocab_size=1000)
