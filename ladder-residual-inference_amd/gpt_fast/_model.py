@@ -162,6 +162,19 @@ class GPTBase(nn.Module):
         raise NotImplementedError
 
     # -- shared pieces of the block schedules -----------------------------------------------------
+    # decode batches from which single projections go to the weight-streaming bands (one row: the matrix-vector kernel
+    # is the faster one -- dense family on the 70B rank shard, ms per step at batch 1 / 4: 5.7 / 8.5 without bands,
+    # 6.1 / 6.2 with)
+    band_rows_from = 2
+
+    def _decode_bands(self, ws: Workspace, *linears) -> bool:
+        """A decode step of up to 64 rows on bf16 weights: every projection of a block is a launch of the
+        weight-streaming kernel (lr_linear_multi), the q/k/v one rotating and caching on its way out and the up/gate one
+        storing silu(gate) * up -- also below 5 rows, where lr_linear alone would pick the matrix-vector kernel: fewer
+        launches per block weigh more than the kernel.  (`linears`: the modules
+        in question; weight-only quantised ones have kernels of their own.)"""
+        return ws.S == 1 and self.band_rows_from <= ws.B <= 64 and not any(hasattr(m, "scales") for m in linears)
+
     def _attention(self, ws: Workspace, blk, pos: Tensor, wqkv: nn.Module, out: Tensor, roped: bool = False):
         """ws.xn -> fused projection -> RoPE + cache write -> attention -> wo -> out (partial sum).
         wqkv None: ws.qkv already holds the projection (roped: rotated, with k and v already in the cache).
@@ -170,7 +183,11 @@ class GPTBase(nn.Module):
         B, S = ws.B, ws.S
         Hq, Hkv, hd = cfg.n_head_local, cfg.n_kv_local, cfg.head_dim
         kc, vc = blk.attention.kv_cache.k_cache, blk.attention.kv_cache.v_cache
-        if wqkv is not None:
+        bands = self._decode_bands(ws, blk.attention.wo, *(() if wqkv is None else (wqkv,)))
+        if wqkv is not None and bands and not roped:
+            _hip.linear_multi((ws.xn, wqkv.weight, ws.qkv, _hip.rope_kv_epilogue(self.freqs_cis, pos, kc, vc, Hq, Hkv, hd)))
+            roped = True
+        elif wqkv is not None:
             _hip.module_linear(ws.xn, wqkv, ws.qkv)
         if not roped:
             _hip.rope_kv_write(ws.qkv, self.freqs_cis, False, pos, kc, vc, B, S, Hq, Hkv, hd)
@@ -178,12 +195,20 @@ class GPTBase(nn.Module):
             _hip.attn_decode(ws.qkv, kc, vc, pos, ws.y, ws.scratch, B, Hq, Hkv, hd)
         else:
             _hip.attn_prefill(ws.qkv, kc, vc, pos, ws.y, B, S, Hq, Hkv, hd)
-        if out is not None:
+        if out is None:
+            return
+        if bands:
+            _hip.linear_multi((ws.y, blk.attention.wo.weight, out, _hip.EPI_NONE))
+        else:
             _hip.module_linear(ws.y, blk.attention.wo, out)
 
     def _mlp(self, ws: Workspace, blk, out: Tensor, xn: Optional[Tensor] = None):
         ff = blk.feed_forward
         xin = ws.xn if xn is None else xn
+        if self._decode_bands(ws, ff.w1, ff.w2):
+            _hip.linear_multi((xin, ff.w1.weight, ws.act, _hip.EPI_SWIGLU))
+            _hip.linear_multi((ws.act, ff.w2.weight, out, _hip.EPI_NONE))
+            return
         if xin.shape[0] > 4 and not hasattr(ff.w1, "scales"):
             # the activation in the first projection's epilogue; up to 4 rows it is fused into w2's GEMV instead
             _hip.linear_swiglu_out(xin, ff.w1.weight, ws.act, ws.h)

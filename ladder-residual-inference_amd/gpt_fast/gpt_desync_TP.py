@@ -59,11 +59,19 @@ class GPTDesync(GPTBase):
     def _run_layers(self, ws: Workspace, pos: Tensor):
         eps = self.config.norm_eps
         tp = float(self.config.tp_world_size)
+        pending = None   # a module output whose residual is not divided: its add rides in the next norm launch
         for blk in self.layers:
-            _hip.add_rmsnorm(ws.x, None, None, blk.attention_norm.weight, None, ws.xn, eps)
+            _hip.add_rmsnorm(ws.x, pending, None, blk.attention_norm.weight, None if pending is None else ws.x, ws.xn,
+                             eps)
             self._attention(ws, blk, pos, blk.attention.wqkv, ws.a)
-            _hip.add(ws.a, ws.x, ws.x, tp if blk.do_attention_all_reduce else 1.0)
-            _hip.add_rmsnorm(ws.x, None, None, blk.ffn_norm.weight, None, ws.xn, eps)
+            pending = ws.a
+            if blk.do_attention_all_reduce and tp != 1.0:
+                _hip.add(ws.a, ws.x, ws.x, tp)
+                pending = None
+            _hip.add_rmsnorm(ws.x, pending, None, blk.ffn_norm.weight, None if pending is None else ws.x, ws.xn, eps)
             self._mlp(ws, blk, ws.m)
-            _hip.add(ws.m, ws.x, ws.x, tp if blk.do_mlp_all_reduce else 1.0)
-        return None, None
+            pending = ws.m
+            if blk.do_mlp_all_reduce and tp != 1.0:
+                _hip.add(ws.m, ws.x, ws.x, tp)
+                pending = None
+        return pending, None

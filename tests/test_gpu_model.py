@@ -699,6 +699,42 @@ def test_variants_on_70b_shard_shape(family):
     check(stats)
 
 
+@pytest.mark.parametrize("family", ["dense", "desync", "parallel"])
+@pytest.mark.parametrize("B", [3, 20])
+@pytest.mark.parametrize("semi", [False, True])
+@torch.no_grad()
+def test_variant_decode_on_the_bands_equals_the_single_projection_kernels(family, B, semi):
+    """Decode steps of the other families through lr_linear_multi (q/k/v with the RoPE + cache epilogue, up/gate with
+    the SwiGLU epilogue; parallel family: up/gate beside the attention up to 16 rows, beside q/k/v above, y + x left to
+    the next norm) against the same steps through lr_linear and the separate kernels: the same tokens fed, logits
+    within the tolerance of two summation orders, KV caches too.  semi: a rank that carries no residual."""
+    kw = dict(TINY, tp_world_size=2, tp_rank=1, semi_compiled_model=semi)
+    if family == "desync":
+        kw.update(reduce_pattern=[{"attention": True, "mlp": False}, {"attention": False, "mlp": True},
+                                  {"attention": False, "mlp": False}])
+    model = build(family, **kw)
+    model.setup_caches(B, 32)
+    g = torch.Generator(device=DEV)
+    g.manual_seed(3)
+    toks = torch.randint(0, 512, (B, 10), device=DEV, generator=g)
+
+    def steps(rows_from):
+        model.band_rows_from = rows_from
+        out = [model(toks[:, :6], torch.arange(6, device=DEV)).clone()]
+        for t in range(6, 10):
+            out.append(model(toks[:, t:t + 1], torch.tensor([t], device=DEV)).clone())
+        model.check_device_errors()
+        kv = model.layers[-1].attention.kv_cache
+        return out, kv.k_cache[:B, :, :10].clone(), kv.v_cache[:B, :, :10].clone()
+
+    plain, kp, vp = steps(10 ** 9)
+    bands, kb, vb = steps(1)
+    assert torch.equal(plain[0], bands[0])   # prefill does not depend on the switch
+    for a, b in zip(plain[1:], bands[1:]):
+        assert rel_err(b, a) <= REL_TOL
+    assert rel_err(kb, kp) <= REL_TOL and rel_err(vb, vp) <= REL_TOL
+
+
 def test_parallel_semi_compiled_nonzero_rank_drops_the_residual():
     """gpt_parallel_TP.py:197-199: in the semi-compiled model only rank 0 adds the residual."""
     kw = dict(TINY, n_layer=2, tp_world_size=2, tp_rank=1, semi_compiled_model=True)
