@@ -31,8 +31,9 @@ Measured in the same run and reported as extra keys (not the headline; --no-extr
 `batched`     : the same rank shard at batch 8 and 64, the 8B model at batch 1 (one-kernel step) and 16 (prompt
                1024) and the 405B rank shard at batch 16 (context 4096) -- per-op kernels unless noted,
                hipGraph replay: ms per step, tok/s, algorithmic GB/s and its fraction of 8 TB/s.
-`fp8`         : the same shard with weight-only e4m3 projections at batch 1 (per-op kernels): ms per
-               step and the fraction of 8 TB/s on ITS algorithmic bytes (one byte per weight + scales).
+`fp8`         : the same shard with weight-only e4m3 projections at batch 1 (the one-kernel step on e4m3 weights)
+               and batch 8 (per-op kernels): ms per step and the fraction of 8 TB/s on ITS algorithmic bytes
+               (one byte per weight + scales).
 `prefill`     : Ladder-8B, batch 32 x 2048 prompt tokens, causal prefill with last-position logits:
                seconds, algorithmic TFLOP/s and the fraction of 2.5 PFLOP/s (dense bf16 MFMA peak)."""
 import argparse
@@ -161,9 +162,11 @@ def extra_fp8(bm, model, prompt, T, K=32, W=5):
 
     quantize_model_fp8(model)
     res = []
-    for B, kernels in ((1, "per-op (fp8 matrix-vector kernel), hipGraph replay"),
+    for B, kernels in ((1, "one-kernel step (lr_ladder_decode_step_fp8), hipGraph replay"),
                        (8, "per-op (fp8 matrix-core bands), hipGraph replay")):
         ms, _, dg = decode_run(bm, model, prompt, B, T, K, W)
+        if B == 1 and model._fused_step(B) is None:
+            kernels = "per-op (fp8 matrix-vector kernel), hipGraph replay"
         nbytes = sum(fp8_bytes_per_step(model.config, B, T + i) for i in range(K)) / K
         gbps = nbytes / (ms * 1e-3) / 1e9
         res.append({"batch": B, "ms_per_step": round(ms, 4), "tok_per_s": round(B * 1e3 / ms, 1),
@@ -293,7 +296,7 @@ def main():
     # ---- dominant kernel, timed with HIP events on the stream it is launched on (torch's current stream)
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     fused = getattr(model, "use_fused_step", False) and hasattr(model, "decode_step_fused") and \
-        model._fused_step(B) is not None and not args.fp8
+        model._fused_step(B) is not None
     if fused:
         # the whole step is ONE kernel (k_ladder_step): algorithmic bytes per launch = bytes per step
         pos = torch.tensor([T], dtype=torch.int32, device=dev)
@@ -309,9 +312,9 @@ def main():
         torch.cuda.synchronize()
         k_us = 1e3 * ev0.elapsed_time(ev1) / reps
         model.check_device_errors()
-        k_bytes = bm.decode_bytes_per_step(cfg, B, T)
+        k_bytes = bytes_per_step(cfg, B, T)
         k_name = (f"k_ladder_step (one persistent launch = the whole decode step at position {T}: "
-                  f"{cfg.n_layer} layers + lm_head, M={B})")
+                  f"{cfg.n_layer} layers + lm_head, M={B}{', e4m3 weights' if args.fp8 else ''})")
     else:
         # per-op path: the weight-streaming GEMV on the w1 (up+gate) projection, a distinct matrix per launch
         w1s = [blk.feed_forward.w1.weight for blk in model.layers] if hasattr(model.layers[0], "feed_forward") else \
@@ -375,7 +378,7 @@ def main():
         "roofline": {"bound": "hbm", "kernel": k_name,
                      "achieved": round(k_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(k_gbps / HBM_PEAK_GBPS, 4),
-                     "traffic": TRAFFIC_BYTES_PER_LAUNCH.get((args.model, B, T)) if fused else None,
+                     "traffic": TRAFFIC_BYTES_PER_LAUNCH.get((args.model, B, T)) if fused and not args.fp8 else None,
                      "bytes_per_launch": int(k_bytes), "avg_launch_us": round(k_us, 3),
                      "measured_read_ceiling": round(ceiling_gbps, 1),
                      "frac_of_measured_ceiling": round(k_gbps / ceiling_gbps, 4)},

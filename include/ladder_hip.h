@@ -339,6 +339,19 @@ int lr_ladder_decode_step(const lr_ladder_model_t* model, int batch, const int32
                           int64_t ld_hist, int hist_len, int pos0, void* workspace, size_t bytes, lr_stream_t stream);
 size_t lr_ladder_step_fail_offset(void);
 
+/* The same step for a weight-only quantised model (every projection of the blocks and the lm_head; the size
+ * accounting of gpt_ladder_TP.py:232-237 is the reference's hook for such layers, it ships no quantised layer):
+ * wqkv / wo / w1 / w2 of lr_layer_t and `output` each point to a matrix of N * K float8_e4m3fn bytes FOLLOWED
+ * IMMEDIATELY by its N bf16 scales (one per output row), and a projection is
+ * bf16(bf16(x . w8^T, fp32 sums) * scales) -- what lr_linear_fp8 computes.  Norm gains, embedding table, RoPE
+ * table and KV caches stay bf16.  Descriptor, workspace (lr_ladder_step_workspace_bytes / lr_ladder_step_init /
+ * lr_ladder_step_fail_offset), arguments and failure reporting are those of lr_ladder_decode_step; in addition
+ * dim, ffn and n_head * head_dim must be multiples of 16 and no matrix may reach 2 GiB (LR_E_UNSUPPORTED). */
+int lr_ladder_decode_step_fp8(const lr_ladder_model_t* model, int batch, const int32_t* tokens, int32_t* pos,
+                              void* logits, int64_t ldl, int32_t* next_token, int advance, int32_t* cur_token,
+                              int32_t* history, int64_t ld_hist, int hist_len, int pos0, void* workspace, size_t bytes,
+                              lr_stream_t stream);
+
 /* benchmark.py:58-77 (sample, logits_to_probs, multinomial_sample_one_no_sync) on the bf16 logits of
  * the last position, one row per sequence: s = bf16(logits * (1 / max(temperature, 1e-5))); values
  * below the top_k-th largest become -inf (top_k <= 0: no cut; top_k > V: V); probs = bf16 softmax

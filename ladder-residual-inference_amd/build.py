@@ -18,6 +18,8 @@ LIB = os.path.join(HERE, "gpt_fast", "libladder_hip.so")
 PROF_LIB = os.path.join(HERE, "gpt_fast", "libladder_hip_prof.so")
 HEADERS = [os.path.join(CSRC, h) for h in ("lr_common.h", "attn_decode_item.h", "stream_band.h")] + \
     [os.path.join(HERE, "..", "include", "ladder_hip.h")]
+# sources that compile another source under a switch
+INCLUDES = {"ladder_step_fp8.hip": [os.path.join(CSRC, "ladder_step.hip")]}
 
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",
@@ -36,7 +38,7 @@ def _stale(target, deps):
 
 def _compile(src, force, extra=(), suffix=""):
     obj = os.path.join(OBJ, os.path.basename(src).replace(".hip", suffix + ".o"))
-    if not force and not _stale(obj, [src] + HEADERS):
+    if not force and not _stale(obj, [src] + HEADERS + INCLUDES.get(os.path.basename(src), [])):
         return obj, False
     cmd = ["hipcc"] + FLAGS + list(extra) + ["-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)

@@ -67,9 +67,25 @@
 // Every retry loop is bounded: on time-out a workgroup raises ctrl->fail and goes on with
 // whatever it has; everybody leaves at the end of the slot in which they see the flag, so the
 // grid always drains.
+// LR_STEP_W8 (ladder_step_fp8.hip compiles this file with it set): the same kernel for weight-only e4m3
+// projections.  A matrix [N, K] is N * K bytes followed by its N bf16 scales (one per output row); a unit is 8 rows x
+// 1 KiB = 1024 elements of K, expanded to packed bf16 pairs (exactly: e4m3 is a subset of bf16) in front of the same
+// v_dot2_f32_bf16; a sum is rounded to bf16, multiplied by its row's scale and rounded again -- what lr_linear_fp8
+// computes.  Only lr_ladder_decode_step_fp8 is exported by that translation unit.
 #include "lr_common.h"
 
+#include <algorithm>
+
+#ifndef LR_STEP_W8
+#define LR_STEP_W8 0
+#endif
+
 namespace {
+
+constexpr bool W8 = LR_STEP_W8 != 0;
+constexpr int KSTEP = W8 ? 1024 : 512;  // elements of K a wave covers per unit (16 bytes per lane and row)
+constexpr int KPL = KSTEP / 64;         // ... per lane
+constexpr int WBYTES = W8 ? 1 : 2;      // bytes per weight
 
 constexpr int NT = 512;           // lanes per workgroup
 constexpr int NW = NT / 64;       // waves per workgroup
@@ -286,6 +302,11 @@ typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ float dot2(u32 a, u32 b, float c) {
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
 }
+// the low (HI == false) or high two e4m3 values of a dword as a packed bf16 pair (exact)
+template <bool HI>
+__device__ __forceinline__ u32 fp8_pair(u32 v) {
+  return __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v, 1.0f, HI));
+}
 
 // ---- per-lane accumulators -> wave totals.  reduce8: afterwards lane 16*r holds sum(v[2r]) in z0
 //      and sum(v[2r+1]) in z1.  (permlane swaps fold halves / odd-even rows, DPP folds a row.)
@@ -366,16 +387,19 @@ struct Job {  // wave-uniform
   int kind;                // JK_*: selects the row-offset table
   const u16* W;            // not in LDS: set per layer
   const int* rowtab;       // not in LDS: row offsets of the first round (see build_row_table)
+#if LR_STEP_W8
+  const u16* S;            // the rows' scales: behind the matrix (table word 15 holds the distance in bytes)
+#endif
 };
-static_assert(sizeof(Job) == 16 * 4 + 16, "16 table words + two pointers");
+static_assert(sizeof(Job) == 16 * 4 + 16 + (W8 ? 8 : 0), "16 table words + two pointers");
 
 __device__ __forceinline__ void build_job(int* rec, int kind, int K, int n_items, int pair_off, int rsh, int w, int nwg,
                                           int wave) {
   Job j;
-  j.K = K; j.K2 = K * 2; j.pair_off = pair_off; j.rsh = rsh; j.w = w; j.nwg = nwg;
+  j.K = K; j.K2 = K * WBYTES; j.pair_off = pair_off; j.rsh = rsh; j.w = w; j.nwg = nwg;
   const int nit = (w >= 0 && n_items > w) ? (n_items - w + nwg - 1) / nwg : 0;
   j.nj = nit << rsh;
-  j.ksteps = (K + 511) >> 9;
+  j.ksteps = (K + KSTEP - 1) / KSTEP;
   j.nkg = j.ksteps < NW ? j.ksteps : NW;
   j.nrg = NW / j.nkg;
   j.rg = wave / j.nkg;
@@ -386,6 +410,7 @@ __device__ __forceinline__ void build_job(int* rec, int kind, int K, int n_items
   j.kind = kind;
   const int* src = reinterpret_cast<const int*>(&j);
   for (int i = 0; i < 16; ++i) rec[i] = src[i];
+  if (W8) rec[15] = (n_items << rsh) * K;  // all rows of the matrix, one byte per weight: where its scales start
 }
 
 // table: [JK_COUNT][NW][16] ints in LDS, filled once per launch
@@ -435,6 +460,9 @@ __device__ __forceinline__ Job load_job(const int* table, int kind, int wave, co
   j.bsh = LR_UNI(d.x); j.active = LR_UNI(d.y); j.K = LR_UNI(d.z); j.kind = kind;
   j.W = W;
   j.rowtab = table + JK_COUNT * NW * 16 + kind * NJMAX;
+#if LR_STEP_W8
+  j.S = reinterpret_cast<const u16*>(reinterpret_cast<const unsigned char*>(W) + LR_UNI(d.w));
+#endif
   return j;
 }
 
@@ -451,9 +479,9 @@ struct Unit {
 // what lets the compiler's wait-count insertion wait for exactly the older unit (vmcnt(RB))
 // instead of for everything in flight.
 __device__ __forceinline__ void load_unit(const Job& job, int j0, int jb, int kk, int lane, Unit& u, bool real) {
-  int k = kk * 512 + lane * 8;
+  int k = kk * KSTEP + lane * KPL;
   k = k < job.K ? k : 0;
-  const int voff = real ? k * 2 : (int)0x80000000;
+  const int voff = real ? k * WBYTES : (int)0x80000000;
   __amdgpu_buffer_rsrc_t br = __builtin_amdgcn_make_buffer_rsrc(const_cast<u16*>(job.W), 0, job.W ? 0x7fffffff : 0, 0x00020000);
   int so[RB];
   if (j0 == 0) {  // first round: the offsets are tabulated (two LDS reads instead of ~10 scalar operations per row)
@@ -570,9 +598,40 @@ __device__ __forceinline__ void consume_unit(const Job& job, const Pos& c, const
 #pragma unroll
       for (int i = 0; i < RB; ++i) acc[m][i] = 0.0f;
   }
-  const int k = c.kk * 512 + lane * 8;
+  const int k = c.kk * KSTEP + lane * KPL;
   const bool kv = k < job.K;
   // weights and inputs stay packed bf16 pairs: one v_dot2_f32_bf16 per pair of products (fp32 sums)
+#if LR_STEP_W8
+  uint4 xp[M][2];
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+    xp[m][0] = kv ? *reinterpret_cast<const uint4*>(x + m * job.K + k) : make_uint4(0, 0, 0, 0);
+    xp[m][1] = kv ? *reinterpret_cast<const uint4*>(x + m * job.K + k + 8) : make_uint4(0, 0, 0, 0);
+  }
+#pragma unroll
+  for (int i = 0; i < RB; ++i) {
+    // dword d of the lane's 16 bytes holds elements 4 d .. 4 d + 3
+    u32 wp[8];
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      wp[2 * d] = fp8_pair<false>(u.r[i][d]);
+      wp[2 * d + 1] = fp8_pair<true>(u.r[i][d]);
+    }
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      float a = acc[m][i];
+      a = dot2(wp[0], xp[m][0].x, a);
+      a = dot2(wp[1], xp[m][0].y, a);
+      a = dot2(wp[2], xp[m][0].z, a);
+      a = dot2(wp[3], xp[m][0].w, a);
+      a = dot2(wp[4], xp[m][1].x, a);
+      a = dot2(wp[5], xp[m][1].y, a);
+      a = dot2(wp[6], xp[m][1].z, a);
+      a = dot2(wp[7], xp[m][1].w, a);
+      acc[m][i] = a;
+    }
+  }
+#else
   uint4 xp[M];
 #pragma unroll
   for (int m = 0; m < M; ++m)
@@ -589,6 +648,7 @@ __device__ __forceinline__ void consume_unit(const Job& job, const Pos& c, const
       acc[m][i] = a;
     }
   }
+#endif
   if (c.kk + job.nkg >= job.ksteps) {
 #pragma unroll
     for (int m = 0; m < M; ++m)
@@ -631,6 +691,16 @@ __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, con
   float acc[M][RB];
   for (int j0 = 0; j0 < job.nj; j0 += NJMAX) {
     const int njb = job.nj - j0 < NJMAX ? job.nj - j0 : NJMAX;
+#if LR_STEP_W8
+    // the scales of the outputs this lane will finish are requested now: their round trip is over when the
+    // round's units have been multiplied
+    float sc0 = 1.0f, sc1 = 1.0f;
+    if (tid < (njb >> job.rsh) * M) {
+      const int it_s = job.w + job.nwg * ((j0 >> job.rsh) + tid / M);
+      sc0 = bf_to_f(job.S[it_s]);
+      if (EPI == EPI_SWIGLU) sc1 = bf_to_f(job.S[it_s + job.pair_off]);
+    }
+#endif
     if (job.active && job.rg < njb) {
       const int up = c.up;
       for (int u = 0; u < up; u += 2) {
@@ -658,6 +728,10 @@ __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, con
         for (int g = 0; g < job.nkg; ++g) t += part[(g * NJMAX + jl * RPI + 1) * M + m];
         s1 = round_bf(t);
       }
+#if LR_STEP_W8
+      s0 = round_bf(s0 * sc0);
+      s1 = round_bf(s1 * sc1);
+#endif
       const int it = job.w + job.nwg * ((j0 >> job.rsh) + jl);
       if (m < p.B) {
         if (EPI == EPI_STORE) coh.st(out_wo + (unsigned)(m * ldo + it), s0, tag);
@@ -1509,6 +1583,13 @@ static int validate(const lr_ladder_model_t* md, int B) {
   const int G = md->n_head / md->n_kv_head;
   if (!has_instance(B, md->head_dim, G)) return LR_E_UNSUPPORTED;
   if (md->n_head * md->head_dim > 16384 || md->ffn > 16384) return LR_E_UNSUPPORTED;
+  if (W8) {
+    // 16 weights per lane and row; a matrix and its scales are addressed with 32-bit byte offsets
+    if (md->dim % 16 || md->ffn % 16 || (md->n_head * md->head_dim) % 16) return LR_E_UNSUPPORTED;
+    const int64_t qkv_rows = (int64_t)(md->n_head + 2 * md->n_kv_head) * md->head_dim;
+    const int64_t most = std::max<int64_t>(std::max<int64_t>(qkv_rows, 2 * (int64_t)md->ffn), md->out_rows) * md->dim;
+    if (most >= 0x7fffffff || (int64_t)md->dim * md->ffn >= 0x7fffffff) return LR_E_UNSUPPORTED;
+  }
   if (lds_need(B, md->head_dim, G, md->dim, md->ffn, md->n_head) > 160 * 1024) return LR_E_UNSUPPORTED;
   const int nwg = num_cus();
   if (nwg < 2) return LR_E_LAUNCH;
@@ -1553,6 +1634,7 @@ extern "C" size_t lr_ladder_step_profile(void* device_buffer, int first_slot) {
 }
 #endif
 
+#if !LR_STEP_W8
 extern "C" size_t lr_ladder_step_workspace_bytes(const lr_ladder_model_t* md, int batch) {
   if (validate(md, batch) != LR_OK) return 0;
   return make_layout(md, batch, num_cus()).total;
@@ -1573,11 +1655,17 @@ extern "C" int lr_ladder_step_init(const lr_ladder_model_t* md, int batch, void*
                                                               (unsigned)(l.total / 4));
   return lr_launch_status();
 }
+#endif
 
-extern "C" int lr_ladder_decode_step(const lr_ladder_model_t* md, int batch, const int32_t* tokens, int32_t* pos,
-                                     void* logits, int64_t ldl, int32_t* next_token, int advance,
-                                     int32_t* cur_token, int32_t* history, int64_t ld_hist, int hist_len, int pos0,
-                                     void* workspace, size_t bytes, lr_stream_t stream) {
+#if LR_STEP_W8
+#define LR_STEP_ENTRY lr_ladder_decode_step_fp8
+#else
+#define LR_STEP_ENTRY lr_ladder_decode_step
+#endif
+extern "C" int LR_STEP_ENTRY(const lr_ladder_model_t* md, int batch, const int32_t* tokens, int32_t* pos,
+                             void* logits, int64_t ldl, int32_t* next_token, int advance,
+                             int32_t* cur_token, int32_t* history, int64_t ld_hist, int hist_len, int pos0,
+                             void* workspace, size_t bytes, lr_stream_t stream) {
   const int rc = validate(md, batch);
   if (rc != LR_OK) return rc;
   LR_REQUIRE_PTR(workspace);

@@ -55,6 +55,8 @@ _PROTOS = {
     "lr_ladder_step_init": (c_int, [c_void_p, c_int, c_void_p, c_size_t, c_void_p]),
     "lr_ladder_decode_step": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_void_p,
                                       c_void_p, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "lr_ladder_decode_step_fp8": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int,
+                                          c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "lr_ladder_step_fail_offset": (c_size_t, []),
 }
 
@@ -521,15 +523,23 @@ def _ladder_model_desc(model, attention_workgroups: int = 0):
     whose addresses they hold."""
     cfg = model.config
     dev = model.output.weight.device
+    fp8 = model.output.weight.dtype == torch.float8_e4m3fn
     rows, keep = [], []
     for blk in model.layers:
-        ts = [blk.attention.wqkv.weight, blk.attention.wo.weight, blk.feed_forward.w1.weight,
-              blk.feed_forward.w2.weight, blk.attention_norm.weight, blk.ffn_norm.weight,
-              blk.attention.kv_cache.k_cache, blk.attention.kv_cache.v_cache]
-        for t in ts:
-            assert t.is_contiguous() and t.dtype == torch.bfloat16 and t.device == dev
-        keep.append(ts)
+        lins = [blk.attention.wqkv, blk.attention.wo, blk.feed_forward.w1, blk.feed_forward.w2]
+        if fp8:
+            for lin in lins:
+                pack_fp8_linear(lin)
+        ts = [lin.weight for lin in lins] + [blk.attention_norm.weight, blk.ffn_norm.weight,
+                                             blk.attention.kv_cache.k_cache, blk.attention.kv_cache.v_cache]
+        for i, t in enumerate(ts):
+            want = torch.float8_e4m3fn if fp8 and i < 4 else torch.bfloat16
+            assert t.is_contiguous() and t.dtype == want and t.device == dev
+        keep.append(ts + ([lin.scales for lin in lins] if fp8 else []))
         rows.append([t.data_ptr() for t in ts])
+    if fp8:
+        pack_fp8_linear(model.output)
+        keep.append(model.output.scales)
     layer_table = torch.tensor(rows, dtype=torch.int64).to(dev)
     keep += [model.tok_embeddings.weight, model.norm.weight, model.output.weight, model.freqs_cis]
     desc = LadderModelDesc(
@@ -540,6 +550,22 @@ def _ladder_model_desc(model, attention_workgroups: int = 0):
         norm=model.norm.weight.data_ptr(), output=model.output.weight.data_ptr(),
         freqs_cis=model.freqs_cis.data_ptr(), layers_dev=layer_table.data_ptr())
     return desc, layer_table, keep
+
+
+def pack_fp8_linear(lin):
+    """The layout lr_ladder_decode_step_fp8 reads: the N bf16 scales of a weight-only e4m3 projection directly behind
+    its N * K weight bytes.  Re-points the module's `weight` and `scales` buffers to views of one allocation (values
+    unchanged) unless they already lie that way."""
+    w, sc = lin.weight, lin.scales
+    N, K = w.shape
+    assert w.dtype == torch.float8_e4m3fn and sc.dtype == torch.bfloat16 and sc.numel() == N and (N * K) % 16 == 0
+    if w.is_contiguous() and sc.is_contiguous() and sc.data_ptr() == w.data_ptr() + N * K and w.data_ptr() % 16 == 0:
+        return
+    buf = _aligned_bytes(N * K + 2 * N, w.device)
+    buf[:N * K].view(torch.float8_e4m3fn).view(N, K).copy_(w)
+    buf[N * K:].view(torch.bfloat16).copy_(sc)
+    lin.weight = buf[:N * K].view(torch.float8_e4m3fn).view(N, K)
+    lin.scales = buf[N * K:].view(torch.bfloat16)
 
 
 def _aligned_bytes(n: int, dev):
@@ -555,11 +581,17 @@ class FusedLadderStep:
 
     def __init__(self, model, batch: int, attention_workgroups: int = 0):
         dev = model.output.weight.device
+        self.fp8 = model.output.weight.dtype == torch.float8_e4m3fn
         self.desc, self.layer_table, self._keep = _ladder_model_desc(model, attention_workgroups)
         self.batch = batch
         lib = load()
         self.bytes = int(lib.lr_ladder_step_workspace_bytes(ctypes.byref(self.desc), batch))
         self.supported = self.bytes > 0
+        if self.fp8:   # the additional conditions of lr_ladder_decode_step_fp8
+            d = self.desc
+            most = max((d.n_head + 2 * d.n_kv_head) * d.head_dim, 2 * d.ffn, d.out_rows) * d.dim
+            self.supported = self.supported and d.dim % 16 == 0 and d.ffn % 16 == 0 and \
+                (d.n_head * d.head_dim) % 16 == 0 and max(most, d.dim * d.ffn) < 0x7fffffff
         self.workspace = None
         if self.supported:
             self.workspace = _aligned_bytes(self.bytes, dev)
@@ -586,7 +618,8 @@ class FusedLadderStep:
         assert lrows == B and lcols == self.desc.out_rows
         p = lambda t: None if t is None else t.data_ptr()
         ld, n = (history.stride(0), history.shape[1]) if history is not None else (0, 0)
-        _check(load().lr_ladder_decode_step(ctypes.byref(self.desc), B, tokens.data_ptr(), pos.data_ptr(),
-                                            logits.data_ptr(), ldl, p(next_token), int(bool(advance)), p(cur_token),
-                                            p(history), ld, n, int(pos0), self.workspace.data_ptr(), self.bytes,
-                                            _stream()), "lr_ladder_decode_step")
+        entry = load().lr_ladder_decode_step_fp8 if self.fp8 else load().lr_ladder_decode_step
+        _check(entry(ctypes.byref(self.desc), B, tokens.data_ptr(), pos.data_ptr(), logits.data_ptr(), ldl,
+                     p(next_token), int(bool(advance)), p(cur_token), p(history), ld, n, int(pos0),
+                     self.workspace.data_ptr(), self.bytes, _stream()),
+               "lr_ladder_decode_step_fp8" if self.fp8 else "lr_ladder_decode_step")

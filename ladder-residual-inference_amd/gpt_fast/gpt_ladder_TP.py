@@ -76,9 +76,12 @@ class GPTLadder(GPTBase):
         if st is None:
             st = self._fused = {}
         if B not in st:
-            # the one-kernel step implements the all-ladder schedule only, on bf16 weights
-            ok = B <= 2 and self.config.ladder_layers is None and self.output.weight.dtype == torch.bfloat16 and \
-                all(p.dtype == torch.bfloat16 for p in self.layers[0].state_dict().values() if p.dim() == 2)
+            # the one-kernel step implements the all-ladder schedule only, on bf16 weights or with every projection
+            # (lm_head included) in weight-only e4m3
+            kinds = {p.dtype for blk in self.layers for p in blk.state_dict().values() if p.dim() == 2}
+            kinds.add(self.output.weight.dtype)
+            ok = B <= 2 and self.config.ladder_layers is None and \
+                kinds in ({torch.bfloat16}, {torch.float8_e4m3fn})
             st[B] = _hip.FusedLadderStep(self, B) if ok else None
             if st[B] is not None and not st[B].supported:
                 st[B] = None

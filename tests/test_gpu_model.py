@@ -334,15 +334,22 @@ STEP_INSTANCES = [(1, 128, 8), (2, 128, 8), (1, 128, 4), (2, 128, 4), (1, 64, 4)
 
 
 @pytest.mark.parametrize("B,hd,G", STEP_INSTANCES)
-def test_fused_step_every_instance(B, hd, G):
+@pytest.mark.parametrize("fp8", [False, True])
+def test_fused_step_every_instance(B, hd, G, fp8):
     """One parity run per (batch, head_dim, q heads per kv head) the step kernel is built for: multi-head
     attention (G = 1, where the shared-memory carve-up has an odd number of per-head scalars), grouped
-    queries up to 16 per kv head, both head sizes."""
+    queries up to 16 per kv head, both head sizes; on bf16 weights and on weight-only e4m3 projections
+    (lr_ladder_decode_step_fp8, against the oracle on the same quantised weights and scales)."""
+    from gpt_fast.quantize import quantize_model_fp8
+
     hkv = 1 if G == 16 else 2
     kw = dict(TINY, block_size=128, n_head=hkv * G, n_local_heads=hkv, dim=hkv * G * hd, intermediate_size=512,
               n_layer=2)
-    stats = run_parity(build("ladder", **kw), "ladder", B=B, T=40, new=6, fused=True)
-    print(B, hd, G, stats)
+    model = build("ladder", **kw)
+    if fp8:
+        quantize_model_fp8(model)
+    stats = run_parity(model, "ladder", B=B, T=40, new=6, fused=True)
+    print(B, hd, G, fp8, stats)
     check(stats)
     assert stats["fused_step_used"]
 
@@ -505,13 +512,56 @@ def test_tiny_models_with_fp8_weights(family):
     stats = run_parity(model, family, B=2, T=20, new=10)
     print(family, stats)
     check(stats)
-    assert not stats["fused_step_used"]
+    assert stats["fused_step_used"] == (family == "ladder")
 
 
-@pytest.mark.parametrize("B", [1, 8])
+@pytest.mark.parametrize("B", [1, 2])
+@torch.no_grad()
+def test_tiny_ladder_fp8_one_kernel_step_against_the_per_op_kernels(B):
+    """lr_ladder_decode_step_fp8 and the per-op fp8 kernels on the same quantised model and the same tokens: logits
+    within the tolerance of two summation orders, the same KV cache rows; a model whose lm_head stays bf16 is not
+    taken by the one-kernel step; packing the scales behind the weights leaves the values as they were."""
+    from gpt_fast.quantize import quantize_model_fp8
+
+    model = quantize_model_fp8(build("ladder", **TINY))
+    w_before = model.layers[1].feed_forward.w1.weight.clone()
+    s_before = model.layers[1].feed_forward.w1.scales.clone()
+    model.setup_caches(B, 32)
+    g = torch.Generator(device=DEV)
+    g.manual_seed(5)
+    toks = torch.randint(0, 512, (B, 12), device=DEV, generator=g)
+
+    def steps(fused):
+        model.use_fused_step = fused
+        out = [model(toks[:, :6], torch.arange(6, device=DEV)).clone()]
+        for t in range(6, 12):
+            out.append(model(toks[:, t:t + 1], torch.tensor([t], device=DEV)).clone())
+        model.check_device_errors()
+        kv = model.layers[-1].attention.kv_cache
+        return out, kv.k_cache[:B, :, :12].clone(), kv.v_cache[:B, :, :12].clone()
+
+    per_op, kp, vp = steps(False)
+    one, ko, vo = steps(True)
+    assert model._fused[B] is not None and model._fused[B].fp8
+    for a, b in zip(per_op, one):
+        assert rel_err(b, a) <= REL_TOL
+    assert rel_err(ko, kp) <= REL_TOL and rel_err(vo, vp) <= REL_TOL
+    w1 = model.layers[1].feed_forward.w1
+    assert torch.equal(w1.weight.view(torch.uint8), w_before.view(torch.uint8)) and torch.equal(w1.scales, s_before)
+    assert w1.scales.data_ptr() == w1.weight.data_ptr() + w1.weight.numel()
+
+    mixed = quantize_model_fp8(build("ladder", **TINY), include_output=False)
+    mixed.setup_caches(B, 32)
+    mixed(toks[:, :6], torch.arange(6, device=DEV))
+    mixed(toks[:, 6:7], torch.tensor([6], device=DEV))
+    assert mixed._fused[B] is None
+
+
+@pytest.mark.parametrize("B", [1, 2, 8])
 def test_ladder_70b_tp8_shard_shape_with_fp8_weights(B):
     """The 70B rank shard's matrices (12 layers) in the weight-only fp8 form: prefill (expanded weights, matrix-core
-    GEMM) and decode (fp8 GEMV) against the oracle on the same fp8 weights and scales."""
+    GEMM) and decode (batch 1 and 2: the one-kernel fp8 step; batch 8: the fp8 bands) against the oracle on the same
+    fp8 weights and scales."""
     from gpt_fast.quantize import quantize_model_fp8
 
     model = quantize_model_fp8(build("ladder", **shape_kw("ladder-70b-tp8", 12)))
