@@ -102,6 +102,7 @@ def test_validation_precedes_any_device_work(lib):
     one8[0].K, one8[0].ldx, one8[0].scales = 16, 16, None
     assert lib.lr_linear_fp8_multi(ptr8, 1, 1, None) == E_NULL
     assert lib.lr_ladder_decode_step(None, 1, None, None, None, 0, None, 0, None, None, 0, 0, 0, None, 0, None) == E_NULL
+    assert lib.lr_ladder_decode_step_fp8(None, 1, None, None, None, 0, None, 0, None, None, 0, 0, 0, None, 0, None) == E_NULL
     assert lib.lr_ladder_step_workspace_bytes(None, 1) == 0
 
 
