@@ -1,11 +1,11 @@
 """Where the time of one decode step of the one-kernel Ladder path goes, per phase of a layer slot.
 
     python build.py --profile-step          # once, anywhere hipcc runs: gpt_fast/libladder_hip_prof.so
-    python step_phases.py [--model gpt_ladder:ladder-70b-tp8] [--prompt 2048] [--slot 40]
+    python step_phases.py [--model gpt_ladder:ladder-70b-tp8] [--prompt 2048] [--slot 40] [--batch 1]
 
 The profile build of the step kernel writes, per workgroup, a 100 MHz wall-clock stamp at every phase boundary of
 four consecutive layer slots (lr_ladder_step_profile, profile builds only).  This script runs a few steps of the
-benchmark workload (random weights, batch 1) on that library and prints, per phase, the mean / min / max duration
+benchmark workload (random weights, batch 1 or 2) on that library and prints, per phase, the mean / min / max duration
 over the workgroups -- attention workgroups and weight-streaming workgroups separately -- the slot length, and
 which workgroups (on which XCD / shader engine / CU) finish the slot last."""
 import argparse
@@ -35,6 +35,7 @@ def main():
     ap.add_argument("--prompt", type=int, default=2048)
     ap.add_argument("--slot", type=int, default=40, help="first of the four layer slots that are stamped")
     ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--batch", type=int, default=1, choices=(1, 2))
     args = ap.parse_args()
 
     prof_lib = os.path.join(HERE, "gpt_fast", "libladder_hip_prof.so")
@@ -45,29 +46,31 @@ def main():
 
     model = bm._load_model(args.model, "cuda", torch.bfloat16, seed=0, verbose=False)
     T = args.prompt
-    model.setup_caches(1, T + 64)
+    B = args.batch
+    model.setup_caches(B, T + 64)
     model.last_logits_only = True
     lib = _hip.load()
     lib.lr_ladder_step_profile.restype = ctypes.c_size_t
     lib.lr_ladder_step_profile.argtypes = [ctypes.c_void_p, ctypes.c_int]
     with torch.no_grad():
         prompt = torch.randint(0, model.config.vocab_size, (T,), device="cuda")
-        first = bm.prefill(model, prompt.view(1, -1), torch.arange(T, device="cuda", dtype=torch.int32), greedy=True).clone()
+        first = bm.prefill(model, prompt.view(1, -1).repeat(B, 1), torch.arange(T, device="cuda", dtype=torch.int32),
+                           greedy=True).clone()
         pos = torch.tensor([T], dtype=torch.int32, device="cuda")
         for _ in range(3):
-            model(first.view(1, 1), pos)
+            model(first.view(B, 1), pos)
         nbytes = lib.lr_ladder_step_profile(None, 0)
         buf = torch.zeros(nbytes // 8, dtype=torch.int64, device="cuda")
         lib.lr_ladder_step_profile(buf.data_ptr(), args.slot)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(args.steps):
-            model(first.view(1, 1), pos)
+            model(first.view(B, 1), pos)
         e1.record()
         torch.cuda.synchronize()
         lib.lr_ladder_step_profile(None, 0)
     model.check_device_errors()
-    print(f"{args.model}, batch 1, position {T}: {e0.elapsed_time(e1) / args.steps:.3f} ms per step (profile build, eager launches)")
+    print(f"{args.model}, batch {B}, position {T}: {e0.elapsed_time(e1) / args.steps:.3f} ms per step (profile build, eager launches)")
     a = buf.cpu().numpy().reshape(-1, 4, 16).astype(np.float64) * 0.01   # [workgroup][slot][stamp] in microseconds
     nwg = a.shape[0]
     s = 1   # second of the four stamped slots
