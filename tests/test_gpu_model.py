@@ -735,8 +735,11 @@ def test_ladder_70b_tp8_shard_config3_full(B):
     check(stats)
 
 
-@pytest.mark.parametrize("family", ["dense", "desync", "parallel"])
-def test_variants_on_70b_shard_shape(family):
+@pytest.mark.parametrize("family,B", [("dense", 2), ("desync", 2), ("parallel", 2), ("dense", 8), ("parallel", 1),
+                                      ("parallel", 8), ("parallel", 20)])
+def test_variants_on_70b_shard_shape(family, B):
+    """The other families on the 70B rank shard's matrices (6 layers) against the oracle; decode runs on the bands of
+    lr_linear_multi (parallel family: up/gate beside the attention at 1, 2 and 8 sequences, beside q/k/v at 20)."""
     kw = shape_kw("ladder-70b-tp8", 6)
     if family == "desync":
         # one layer of each kind: no reduce, a reduce after attention (residual / tp), after the MLP, after both
@@ -744,8 +747,8 @@ def test_variants_on_70b_shard_shape(family):
                                   {"attention": False, "mlp": True}, {"attention": True, "mlp": True},
                                   {"attention": False, "mlp": False}, {"attention": False, "mlp": False}],
                   force_disable_last_all_reduce=True)
-    stats = run_parity(build(family, **kw), family, B=2, T=300, new=10)
-    report(f"{family} on the 70B shard shape", stats)
+    stats = run_parity(build(family, **kw), family, B=B, T=300, new=10)
+    report(f"{family} on the 70B shard shape, B={B}", stats)
     check(stats)
 
 
