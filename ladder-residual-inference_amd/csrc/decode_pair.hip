@@ -36,7 +36,7 @@ struct AttnItems {
 
 constexpr int PAIR_MT = 16, PAIR_UNITS = 2;
 
-template <int HD, int G, bool W8>
+template <int HD, int G, bool W8, bool XL>
 __global__ __launch_bounds__(256) void k_attn_beside_band(const AttnItems a, const Proj p, const int M) {
   extern __shared__ __attribute__((aligned(16))) unsigned char pair_smem[];
   const int wg = blockIdx.x;
@@ -46,24 +46,31 @@ __global__ __launch_bounds__(256) void k_attn_beside_band(const AttnItems a, con
                              a.chunk_max, split, rest % a.Hkv, rest / a.Hkv, reinterpret_cast<float*>(pair_smem),
                              a.kv_share);
   } else {
-    stream_band<PAIR_MT, PAIR_UNITS, W8>(p, M, wg - a.n_items, reinterpret_cast<u16*>(pair_smem));
+    stream_band<PAIR_MT, PAIR_UNITS, W8, XL>(p, M, wg - a.n_items, reinterpret_cast<u16*>(pair_smem));
   }
 }
 
-template <int HD, int G, bool W8>
-static int launch_pair(const AttnItems& a, const Proj& p, int M, u16* y, int64_t ldy, int B, hipStream_t s) {
+template <int HD, int G, bool W8, bool XL>
+static int launch_pair_as(const AttnItems& a, const Proj& p, int M, u16* y, int64_t ldy, int B, hipStream_t s) {
   const int Hq = a.Hkv * G;
   const size_t lds_att = (size_t)attn_item_lds_floats<HD, G>(a.chunk_max) * sizeof(float);
-  const size_t lds_band = stream_band_lds_bytes<PAIR_MT, PAIR_UNITS, W8>();
+  const size_t lds_band = stream_band_lds_bytes<PAIR_MT, PAIR_UNITS, W8, XL>();
   const size_t lds = lds_att > lds_band ? lds_att : lds_band;
   if (lds > 64 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_attn_beside_band<HD, G, W8>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_attn_beside_band<HD, G, W8, XL>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return LR_E_LAUNCH;
   }
-  k_attn_beside_band<HD, G, W8><<<dim3((unsigned)(a.n_items + p.nwg)), dim3(256), lds, s>>>(a, p, M);
+  k_attn_beside_band<HD, G, W8, XL><<<dim3((unsigned)(a.n_items + p.nwg)), dim3(256), lds, s>>>(a, p, M);
   k_attn_decode_combine<HD><<<dim3(Hq, B), dim3(HD), 0, s>>>(a.o_part, a.ml_part, y, ldy, Hq, a.nsplit);
   return lr_launch_status();
+}
+
+// (the band's inputs in whole lines or in fragment layout: the choice lr_linear_multi makes for the same rows)
+template <int HD, int G, bool W8>
+static int launch_pair(const AttnItems& a, const Proj& p, int M, u16* y, int64_t ldy, int B, hipStream_t s) {
+  if (!W8 && M >= LR_SG_XLDS_M16_FROM) return launch_pair_as<HD, G, false, true>(a, p, M, y, ldy, B, s);
+  return launch_pair_as<HD, G, W8, false>(a, p, M, y, ldy, B, s);
 }
 
 // shared body of the two entry points; `fill` turns the caller's projection into a Proj

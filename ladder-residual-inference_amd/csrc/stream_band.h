@@ -11,8 +11,15 @@ constexpr int NWV = 4;         // waves per workgroup
 constexpr int SETS = 4;        // weight chunks in flight per wave
 constexpr int LROW = KC + 8;   // LDS row length in elements (272 bytes)
 constexpr int OOB = (int)0x80000000;  // a buffer offset beyond every resource: the load returns zero, untouched memory
+// Input rows from which a band reads the inputs in whole cache lines (through LDS) rather than in fragment layout:
+// always with the 32- and 64-row bands; the 16-row band has both forms and the launcher picks by the row count
+// (70B rank shard, ms per step, fragment layout / whole lines: 4 rows 4.99 / 5.12, 8 rows 5.14 / 5.19, 16 rows
+// 6.26 / 6.00; 8B, 16 rows: 4.00 / 3.78)
 #ifndef LR_SG_XLDS_MIN
 #define LR_SG_XLDS_MIN 32
+#endif
+#ifndef LR_SG_XLDS_M16_FROM
+#define LR_SG_XLDS_M16_FROM 9
 #endif
 #ifndef LR_SG_W_AUX
 #define LR_SG_W_AUX 2          // weights: non-temporal (every line is used exactly once)
@@ -43,10 +50,10 @@ __device__ __forceinline__ u32 sb_fp8_pair(u32 v) {
   return __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v, 1.0f, HI));
 }
 
-template <int MT, int UNITS, bool W8 = false>
+template <int MT, int UNITS, bool W8 = false, bool XL = (MT >= LR_SG_XLDS_MIN)>
 constexpr size_t stream_band_lds_bytes() {
   constexpr int LRW = (W8 ? 2 * KC : KC) + 8;
-  return (size_t)NWV * (UNITS * 16 * LRW + (MT >= LR_SG_XLDS_MIN ? MT * LRW : 0)) * sizeof(u16);
+  return (size_t)NWV * (UNITS * 16 * LRW + (XL ? MT * LRW : 0)) * sizeof(u16);
 }
 
 // One band of one projection, by the 256 lanes of a workgroup.  `sg_smem`: stream_band_lds_bytes<MT, UNITS>() bytes of LDS.
@@ -54,7 +61,7 @@ constexpr size_t stream_band_lds_bytes() {
 // 256 bytes, now 256 elements of K, which are expanded to bf16 (exactly: e4m3 is a subset of bf16) on their way
 // into the LDS piece; the sum is rounded to bf16, multiplied by the row's scale and rounded again, as
 // F.linear(x, w.to(bf16)) * scales does, before the epilogue sees it.
-template <int MT, int UNITS, bool W8 = false>
+template <int MT, int UNITS, bool W8 = false, bool XL = (MT >= LR_SG_XLDS_MIN)>
 __device__ __forceinline__ void stream_band(const Proj& p, const int M, const int band, u16* sg_smem) {
   static_assert(!W8 || MT == 16, "the e4m3 path is built for up to 16 input rows");
   constexpr int KCW = W8 ? 256 : 128;  // k elements per chunk
@@ -68,10 +75,11 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
   constexpr int NS = W8 ? LR_SG_W8_SETS : SETS;
   constexpr int MTILES = MT / 16, KS = KCW / 32, NLD = UNITS * 4;
   constexpr int NV = UNITS * MTILES * 4;  // accumulator registers per lane
-  // From 32 input rows on the inputs too are loaded in whole lines (4 rows x 256 bytes per instruction) and take
-  // the trip through LDS into B-fragment layout: L2 serves whole-line reads 1.5 times as fast as the 16 rows x
-  // 64 bytes a fragment-layout load touches, and at 64 rows the input bytes are twice the weight bytes.
-  constexpr bool XLDS = MT >= LR_SG_XLDS_MIN;
+  // XL: the inputs too are loaded in whole lines (4 rows x 256 bytes per instruction) and take the trip through
+  // LDS into B-fragment layout: L2 serves whole-line reads 1.5 times as fast as the 16 rows x 64 bytes a
+  // fragment-layout load touches, and at 64 rows the input bytes are twice the weight bytes.
+  constexpr bool XLDS = XL;
+  static_assert(!(XL && W8), "the e4m3 band reads its inputs in fragment layout");
   constexpr int WPIECE = UNITS * 16 * LRW, XPIECE = XLDS ? MT * LRW : 0;  // elements per wave
   // sg_smem: [NWV][WPIECE + XPIECE]
   static_assert(sizeof(float) * NV * 64 <= sizeof(u16) * WPIECE, "the partial sums reuse the wave's weight piece");

@@ -24,30 +24,32 @@
 
 namespace {
 
-template <int MT, int UNITS, bool W8>
+template <int MT, int UNITS, bool W8, bool XL>
 __global__ __launch_bounds__(NWV * 64) void k_stream_gemm(const Proj p0, const Proj p1, const int M) {
   extern __shared__ __attribute__((aligned(16))) u16 sg_smem[];
   const bool second = (int)blockIdx.x >= p0.nwg;
   const Proj p = second ? p1 : p0;
-  stream_band<MT, UNITS, W8>(p, M, second ? (int)blockIdx.x - p0.nwg : (int)blockIdx.x, sg_smem);
+  stream_band<MT, UNITS, W8, XL>(p, M, second ? (int)blockIdx.x - p0.nwg : (int)blockIdx.x, sg_smem);
 }
 
-template <int MT, int UNITS, bool W8 = false>
+template <int MT, int UNITS, bool W8 = false, bool XL = (MT >= LR_SG_XLDS_MIN)>
 static int launch_units(Proj& a, Proj& b, int M, hipStream_t s) {
-  constexpr size_t lds = stream_band_lds_bytes<MT, UNITS, W8>();
+  constexpr size_t lds = stream_band_lds_bytes<MT, UNITS, W8, XL>();
   static bool attr_set = false;
   if (!attr_set && lds > 64 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_stream_gemm<MT, UNITS, W8>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_stream_gemm<MT, UNITS, W8, XL>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return LR_E_LAUNCH;
     attr_set = true;
   }
-  k_stream_gemm<MT, UNITS, W8><<<dim3((unsigned)(a.nwg + b.nwg)), dim3(NWV * 64), lds, s>>>(a, b, M);
+  k_stream_gemm<MT, UNITS, W8, XL><<<dim3((unsigned)(a.nwg + b.nwg)), dim3(NWV * 64), lds, s>>>(a, b, M);
   return LR_OK;
 }
 
 template <int MT>
 static int launch(Proj& a, Proj& b, int M, int units, hipStream_t s) {
+  if (MT == 16 && M >= LR_SG_XLDS_M16_FROM)  // the 16-row band with its inputs read in whole lines
+    return units == 2 ? launch_units<MT, 2, false, true>(a, b, M, s) : launch_units<MT, 1, false, true>(a, b, M, s);
   return units == 2 ? launch_units<MT, 2>(a, b, M, s) : launch_units<MT, 1>(a, b, M, s);
 }
 
