@@ -94,16 +94,10 @@ constexpr int RB = 8;  // rows per unit (loads a wave issues together)
 constexpr unsigned SPIN_LIMIT = 1u << 18;
 constexpr int ATT_NI = 9;         // key iterations an attention wave keeps in registers
 constexpr int NA_MAX = 16;        // attention workgroups (each merges a share of the outputs)
-constexpr int PROF_SLOTS = 4, PROF_POINTS = 16;
+constexpr int PROF_SLOTS = 4, PROF_POINTS = 32;
 // Buffer cache policies (the `aux` operand of the raw buffer builtins: bit 0 sc0, bit 1 nt, bit 4 sc1).
-#ifndef LR_AUX_ST
-#define LR_AUX_ST 16
-#endif
-constexpr int AUX_SC1 = LR_AUX_ST;  // exchange stores: written through, visible to every XCD
-#ifndef LR_AUX_LD
-#define LR_AUX_LD 17
-#endif
-constexpr int AUX_LD = LR_AUX_LD;   // exchange loads: sc0 sc1, never served from a per-XCD L2 line
+// (exchange stores carry sc1 -- written through, visible to every XCD -- in their assembler text, see Coh)
+constexpr int AUX_LD = 17;   // exchange loads: sc0 sc1, never served from a per-XCD L2 line
 constexpr int AUX_W = 2;     // weight loads: non-temporal (measured: nt on the exchange words' loads or stores is far slower)
 constexpr int POLL_SLEEP = 2;
 
@@ -175,9 +169,39 @@ __device__ __forceinline__ unsigned tag_of(unsigned epoch) { return epoch % 6553
 struct Coh {
   __amdgpu_buffer_rsrc_t r;
   unsigned* fail;
+#ifdef LR_STEP_PROFILE
+  // profile builds count, per exchange point, the words that had not arrived at the first look
+  mutable unsigned long long* cnt = nullptr;
+  mutable int where = 24;
+  __device__ __forceinline__ void stale() const {
+    if (cnt) atomicAdd(cnt + where, 1ull);
+  }
+  __device__ __forceinline__ void at(unsigned long long* c, int w) const { cnt = c; where = w; }
+#else
+  __device__ __forceinline__ void stale() const {}
+  __device__ __forceinline__ void at(unsigned long long*, int) const {}
+#endif
 
+  // Exchange stores are written as inline assembly: the compiler's wait-count insertion does not see them.
+  // With a store of its own pending, it must assume that loads and stores complete in any order and waits
+  // for EVERYTHING in flight (vmcnt(0)) wherever a loaded value is used -- also for the weight units requested
+  // for later.  Unseen stores only ever make a counted wait longer than needed, never shorter: if at most N
+  // operations may be outstanding and the N younger loads the compiler counted are joined by a store, one
+  // more operation has to finish, and loads finish in order.
+  // (The scalar words of the resource may have been restored from a lane of a vector register one instruction
+  // earlier; the assembler text is opaque to the hazard recogniser, hence the s_nop in front of every store.)
+  u32x4_t rs;  // the same buffer resource as `r`, as four scalar words
+  __device__ __forceinline__ void st_raw(unsigned word, unsigned byte_off) const {
+    asm volatile("s_nop 4\n\tbuffer_store_dword %0, %1, %2, 0 offen sc1" ::"v"(word), "v"(byte_off), "s"(rs) : "memory");
+  }
+  __device__ __forceinline__ void st_raw2(u32x2_t w, unsigned byte_off) const {
+    asm volatile("s_nop 4\n\tbuffer_store_dwordx2 %0, %1, %2, 0 offen sc1\n\ts_nop 1" ::"v"(w), "v"(byte_off), "s"(rs) : "memory");
+  }
+  __device__ __forceinline__ void st_raw4(u32x4_t w, unsigned byte_off) const {
+    asm volatile("s_nop 4\n\tbuffer_store_dwordx4 %0, %1, %2, 0 offen sc1\n\ts_nop 1" ::"v"(w), "v"(byte_off), "s"(rs) : "memory");
+  }
   __device__ __forceinline__ void st(unsigned wo, float v, unsigned tag) const {  // v is bf16-representable
-    __builtin_amdgcn_raw_buffer_store_b32((__float_as_uint(v) & 0xffff0000u) | tag, r, wo * 4, 0, AUX_SC1);
+    st_raw((__float_as_uint(v) & 0xffff0000u) | tag, wo * 4);
   }
   __device__ __forceinline__ void st8(unsigned wo, const float* f, unsigned tag) const {  // wo % 4 == 0
     u32x4_t a, b;
@@ -185,15 +209,15 @@ struct Coh {
     a.z = (__float_as_uint(f[2]) & 0xffff0000u) | tag; a.w = (__float_as_uint(f[3]) & 0xffff0000u) | tag;
     b.x = (__float_as_uint(f[4]) & 0xffff0000u) | tag; b.y = (__float_as_uint(f[5]) & 0xffff0000u) | tag;
     b.z = (__float_as_uint(f[6]) & 0xffff0000u) | tag; b.w = (__float_as_uint(f[7]) & 0xffff0000u) | tag;
-    __builtin_amdgcn_raw_buffer_store_b128(a, r, wo * 4, 0, AUX_SC1);
-    __builtin_amdgcn_raw_buffer_store_b128(b, r, wo * 4 + 16, 0, AUX_SC1);
+    st_raw4(a, wo * 4);
+    st_raw4(b, wo * 4 + 16);
   }
   // two bf16-representable values as two words at wo, wo + 1 (wo % 2 == 0)
   __device__ __forceinline__ void st2(unsigned wo, float v0, float v1, unsigned tag) const {
     u32x2_t w;
     w.x = (__float_as_uint(v0) & 0xffff0000u) | tag;
     w.y = (__float_as_uint(v1) & 0xffff0000u) | tag;
-    __builtin_amdgcn_raw_buffer_store_b64(w, r, wo * 4, 0, AUX_SC1);
+    st_raw2(w, wo * 4);
   }
   // fp32 value as two words at wo, wo + 1 (wo % 2 == 0)
   __device__ __forceinline__ void st_f32(unsigned wo, float v, unsigned tag) const {
@@ -201,7 +225,7 @@ struct Coh {
     u32x2_t w;
     w.x = (bits & 0xffff0000u) | tag;
     w.y = (bits << 16) | tag;
-    __builtin_amdgcn_raw_buffer_store_b64(w, r, wo * 4, 0, AUX_SC1);
+    st_raw2(w, wo * 4);
   }
   __device__ __forceinline__ bool give_up(unsigned& spins) const {
     if ((++spins & 255u) == 0) {
@@ -257,10 +281,12 @@ struct Coh {
   }
   __device__ __forceinline__ u32x4_t settle4(unsigned wo, unsigned tag, const u32x4_t& a) const {
     if ((((a.x ^ tag) | (a.y ^ tag) | (a.z ^ tag) | (a.w ^ tag)) & 0xffffu) == 0) return a;
+    stale();
     return poll4(wo, tag);
   }
   __device__ __forceinline__ u32x2_t settle2(unsigned wo, unsigned tag, const u32x2_t& a) const {
     if ((((a.x ^ tag) | (a.y ^ tag)) & 0xffffu) == 0) return a;
+    stale();
     return poll2(wo, tag);
   }
   // 8 bf16-valued words -> 8 floats
@@ -278,6 +304,7 @@ struct Coh {
         f[6] = __uint_as_float(b.z & 0xffff0000u); f[7] = __uint_as_float(b.w & 0xffff0000u);
         return;
       }
+      if (spins == 0) stale();
       __builtin_amdgcn_s_sleep(POLL_SLEEP);
     }
   }
@@ -336,6 +363,15 @@ __device__ __forceinline__ float half_row_sum8(float r) {  // every lane of an 8
   r += dpp_mov<0xb1>(r);
   r += dpp_mov<0x141>(r);  // row_half_mirror
   return r;
+}
+// sum over the 64 lanes without the LDS crossbar: DPP inside the 16-lane rows, the four row totals through scalar registers
+__device__ __forceinline__ float wave_sum_fast(float v) {
+  const float r = row_sum16(v);
+  const float a = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(r), 0));
+  const float b = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(r), 16));
+  const float c = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(r), 32));
+  const float d = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(r), 48));
+  return (a + b) + (c + d);
 }
 __device__ __forceinline__ void reduce8(float* v, float& z0, float& z1) {
   float w[4];
@@ -671,7 +707,8 @@ __device__ __forceinline__ void consume_unit(const Job& job, const Pos& c, const
 template <int M, int EPI>
 __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, const Job& job, const Job& next,
                                         Pipe& pipe, const u16* x, float* part, unsigned out_wo, int ldo, unsigned tag,
-                                        float* cand_v, int* cand_i, float* best_v, int* best_i) {
+                                        float* cand_v, int* cand_i, float* best_v, int* best_i,
+                                        unsigned long long* stamp = nullptr, int sb = 0) {
   const int tid = opaque_tid(), lane = tid & 63;
   const int RPI = 1 << job.rsh;
   if (!job.active) prime(next, lane, pipe);
@@ -713,20 +750,27 @@ __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, con
       }
     }
     wg_sync();
+    if (stamp && tid == 0) stamp[sb] = wall_clock64();
     // ---- cross-wave sum in fixed order + epilogue
     const int nout = (njb >> job.rsh) * M;
     if (tid < nout) {
       const int jl = tid / M, m = tid - jl * M;
       float s0, s1 = 0.0f;
-      {
-        float t = 0.0f;
-        for (int g = 0; g < job.nkg; ++g) t += part[(g * NJMAX + jl * RPI) * M + m];
+      {  // all partial sums are requested at once; they are added in the same fixed order
+        float v0[NW], v1[NW];
+#pragma unroll
+        for (int g = 0; g < NW; ++g) {
+          v0[g] = part[(g * NJMAX + jl * RPI) * M + m];
+          if (EPI == EPI_SWIGLU) v1[g] = part[(g * NJMAX + jl * RPI + 1) * M + m];
+        }
+        float t = 0.0f, t1 = 0.0f;
+#pragma unroll
+        for (int g = 0; g < NW; ++g) {
+          t = g < job.nkg ? t + v0[g] : t;
+          if (EPI == EPI_SWIGLU) t1 = g < job.nkg ? t1 + v1[g] : t1;
+        }
         s0 = round_bf(t);
-      }
-      if (EPI == EPI_SWIGLU) {
-        float t = 0.0f;
-        for (int g = 0; g < job.nkg; ++g) t += part[(g * NJMAX + jl * RPI + 1) * M + m];
-        s1 = round_bf(t);
+        if (EPI == EPI_SWIGLU) s1 = round_bf(t1);
       }
 #if LR_STEP_W8
       s0 = round_bf(s0 * sc0);
@@ -753,6 +797,7 @@ __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, con
       }
     }
     wg_sync();
+    if (stamp && tid == 0) stamp[sb + 1] = wall_clock64();
   }
 }
 
@@ -803,7 +848,7 @@ __device__ __forceinline__ void residual_step(const StepParams& p, const Coh& co
 #pragma unroll
   for (int it = 0; it < PRO_NIT; ++it) {
     const int c = (it * NT + tid) * 8;
-    gq[it] = (gain && c < D) ? ld16(gain + c) : make_uint4(0, 0, 0, 0);
+    gq[it] = (gain && c < D) ? gld16(gain + c) : make_uint4(0, 0, 0, 0);
   }
   // pass 1: the (bf16-exact) sums go to LDS unscaled; sums of squares per lane
 #pragma unroll
@@ -835,7 +880,7 @@ __device__ __forceinline__ void residual_step(const StepParams& p, const Coh& co
         if (emb_rows) {
           const int id = emb_rows[m];
           const bool ok = id >= 0 && id < p.vocab;
-          unpack8(ok ? ld16(p.tok_emb + (int64_t)id * D + c) : make_uint4(0, 0, 0, 0), v);
+          unpack8(ok ? gld16(p.tok_emb + (int64_t)id * D + c) : make_uint4(0, 0, 0, 0), v);
         } else {
           unpack8(*reinterpret_cast<const uint4*>(xr + m * D + c), v);
         }
@@ -858,16 +903,16 @@ __device__ __forceinline__ void residual_step(const StepParams& p, const Coh& co
       }
     }
   }
-  // The first weight units of the coming job are requested only now, behind the exchange words: a
-  // wave's loads return in order and a CU serves them at a bounded rate, so requested earlier they
-  // would stand between this phase and the words it waits for; from here they travel while the
-  // norm is finished.
+  // The first weight units of the coming job are requested only now, when the exchange words have arrived.
+  // Requested earlier -- right behind the word requests, with the bookkeeping done while the words travel -- the
+  // words come back later and the step is slower (measured, with exact wait counts): every workgroup then sends
+  // its 128 KiB of requests at the moment all of them wait for the words.
   if (stamp && tid == 0) stamp[13] = wall_clock64();
   if (do_prime) prime(first, tid & 63, pipe);
   if (stamp && tid == 0) stamp[15] = wall_clock64();
   if (gain == nullptr) return;  // uniform: only the residual was wanted (each lane revisits its own elements later)
 #pragma unroll
-  for (int m = 0; m < M; ++m) ss[m] = wave_sum(ss[m]);
+  for (int m = 0; m < M; ++m) ss[m] = wave_sum_fast(ss[m]);
   if ((tid & 63) == 0) {
 #pragma unroll
     for (int m = 0; m < M; ++m) red[(tid >> 6) * M + m] = ss[m];
@@ -945,13 +990,13 @@ __device__ __forceinline__ void attention_load(const StepParams& p, const LayerP
     const bool live = key < k1 && key != pos;  // the slot of `pos` is filled from this step's qkv
 #pragma unroll
     for (int s = 0; s < HD / 16; ++s)
-      kv.k[t][s] = live ? ld16(kbase + (int64_t)key * HD + s * 16 + (lane >> 5) * 8) : make_uint4(0, 0, 0, 0);
+      kv.k[t][s] = live ? gld16(kbase + (int64_t)key * HD + s * 16 + (lane >> 5) * 8) : make_uint4(0, 0, 0, 0);
   }
 #pragma unroll
   for (int i = 0; i < ATT_NI; ++i) {
     const int key = k0 + (i * NW + wave) * KPW + kl;
     const bool live = key < k1 && key != pos;
-    kv.v[i] = live ? ld16(vbase + (int64_t)key * HD + dl) : make_uint4(0, 0, 0, 0);
+    kv.v[i] = live ? gld16(vbase + (int64_t)key * HD + dl) : make_uint4(0, 0, 0, 0);
   }
 }
 
@@ -1007,8 +1052,8 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
     kp[j] = pack_bf2(r0, r1);
     vnew[2 * j] = v0; vnew[2 * j + 1] = v1;
     const int64_t slot = (((int64_t)b * Hkv + kvh) * p.Smax + pos) * HD + 2 * j;
-    *reinterpret_cast<u32*>(lp.k_cache + slot) = pack_bf2(r0, r1);
-    *reinterpret_cast<u32*>(lp.v_cache + slot) = pack_bf2(v0, v1);
+    gst4(lp.k_cache + slot, pack_bf2(r0, r1));
+    gst4(lp.v_cache + slot, pack_bf2(v0, v1));
   }
   wg_sync();
   if (stamp && tid == 0) stamp[10] = wall_clock64();
@@ -1222,6 +1267,13 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
   Ctrl* ctrl = reinterpret_cast<Ctrl*>(p.ws);
   Coh coh;
   coh.r = __builtin_amdgcn_make_buffer_rsrc(p.ws, 0, (int)p.ws_bytes, 0x00020000);
+  {
+    const unsigned long long base = reinterpret_cast<unsigned long long>(p.ws);
+    coh.rs.x = LR_UNI((unsigned)base);
+    coh.rs.y = LR_UNI((unsigned)(base >> 32) & 0xffffu);
+    coh.rs.z = LR_UNI(p.ws_bytes);
+    coh.rs.w = 0x00020000u;
+  }
   coh.fail = &ctrl->fail;
   if (tid == 0) {
     s_flag[1] = (int)cldu(&ctrl->epoch_base);
@@ -1311,13 +1363,15 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
       // (no weight units are requested across the attention phase: it is where registers are scarcest, and
       // the attention workgroups are done well before the others have streamed w1)
       run_job<M, EPI_STORE>(p, coh, j_qkv, no_job, pipe, xa, part, p.oqkv, p.nqkv, tag, nullptr, nullptr, nullptr,
-                            nullptr);
+                            nullptr, LR_STAMP_PTR, 16);
       LR_STAMP(2)
+      coh.at(LR_STAMP_PTR, 25);
       // ---------------- attention workgroup (it owns no rows of w1): R += m(t-1) while q is on its way
       if (t >= 1)
         residual_step<M>(p, coh, xr, nullptr, true, p.om, tag_prev, true, ew, false, 0u, 0u, nullptr, xb, red, false,
                          no_job, pipe);
       LR_STAMP(3)
+      coh.at(LR_STAMP_PTR, 28);
       KV<HD> kv;
       LayerPtrs lcache;  // only the cache pointers are used
       lcache.k_cache = const_cast<u16*>(ring_ptr(lring, t, LP_K_CACHE));
@@ -1330,33 +1384,38 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
                                       reinterpret_cast<u32*>(qs), sc, sc_ld, ored, reinterpret_cast<u32*>(knew), vnew,
                                       s_m, s_l);
         }
+      coh.at(LR_STAMP_PTR, 29);
       attention_merge_slice<M, HD>(p, coh, Hq, tag, wbuf, w);
       prime(LR_JOB(JK_WO, LP_WO), opaque_tid() & 63, pipe);
     } else {
       const Job j_w1 = LR_JOB(JK_W1_SPLIT, LP_W1);
       run_job<M, EPI_STORE>(p, coh, j_qkv, j_w1, pipe, xa, part, p.oqkv, p.nqkv, tag, nullptr, nullptr, nullptr,
-                            nullptr);
+                            nullptr, LR_STAMP_PTR, 16);
       LR_STAMP(2)
+      coh.at(LR_STAMP_PTR, 25);
       // ---------------- everyone else: R += m(t-1); ffn norm; the up/gate projection + SwiGLU
       residual_step<M>(p, coh, xr, nullptr, t >= 1, p.om, tag_prev, t >= 1, ew, false, 0u, 0u,
                        ring_ptr(lring, t, LP_FFN_NORM), xb, red, false, no_job, pipe);
       LR_STAMP(3)
       run_job<M, EPI_SWIGLU>(p, coh, j_w1, LR_JOB(JK_WO, LP_WO), pipe, xb, part, act_wo, I, tag, nullptr, nullptr, nullptr,
-                             nullptr);
+                             nullptr, LR_STAMP_PTR, 18);
     }
     LR_STAMP(4)
     // ---------------- merged attention output (published by the attention workgroups), output projection
+    coh.at(LR_STAMP_PTR, 26);
     load_x<M>(coh, p.oy, tag, qdim, xa);
     LR_STAMP(5)
     run_job<M, EPI_STORE>(p, coh, LR_JOB(JK_WO, LP_WO), LR_JOB(JK_W2, LP_W2), pipe, xa, part, p.oa, D, tag, nullptr,
-                          nullptr, nullptr, nullptr);
+                          nullptr, nullptr, nullptr, LR_STAMP_PTR, 20);
     LR_STAMP(6)
     // ---------------- down projection
+    coh.at(LR_STAMP_PTR, 27);
     load_x<M>(coh, act_wo, tag, I, xb);
     LR_STAMP(7)
     run_job<M, EPI_STORE>(p, coh, LR_JOB(JK_W2, LP_W2), no_job, pipe, xb, part, p.om, D, tag, nullptr, nullptr, nullptr,
-                          nullptr);
+                          nullptr, LR_STAMP_PTR, 22);
     LR_STAMP(8)
+    coh.at(LR_STAMP_PTR, 24);
     // ---------------- slot t + 1 opens: R += a(t); attention norm; the first weight units of wqkv(t + 1) go out
     //                  behind the a words.  After the last layer: x = (R + a(L-1)) + m(L-1), the final norm and
     //                  the first units of the lm_head instead.
@@ -1541,13 +1600,9 @@ static Layout make_layout(const lr_ladder_model_t* md, int B, int nwg) {
 }
 
 // (batch, head_dim, q heads per kv head) combinations the step kernel is instantiated for
-#ifdef LR_STEP_ONLY_70B  // experiments: one instance compiles in a fraction of the time
-#define LR_STEP_INSTANCES(X) X(1, 128, 8)
-#else
 #define LR_STEP_INSTANCES(X) \
   X(1, 128, 8) X(2, 128, 8) X(1, 128, 4) X(2, 128, 4) X(1, 64, 4) X(2, 64, 4) X(1, 128, 16) \
   X(1, 64, 2) X(2, 64, 2) X(1, 128, 2) X(1, 128, 1) X(1, 64, 1) X(1, 64, 8)
-#endif
 
 static bool has_instance(int B, int hd, int G) {
 #define LR_HAS(MV, HDV, GV) if (B == MV && hd == HDV && G == GV) return true;

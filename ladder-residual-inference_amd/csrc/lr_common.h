@@ -34,6 +34,19 @@ __device__ __forceinline__ u32 pack_bf2(float lo, float hi) { return (u32)f_to_b
 __device__ __forceinline__ float round_bf(float f) { return bf_to_f(f_to_bf(f)); }
 
 __device__ __forceinline__ uint4 ld16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
+// The same through pointers the compiler cannot trace back to a kernel argument (read from a table, chosen between
+// two sources): stated to be global memory.  A generic ("flat") access could also target LDS, so it counts as an
+// LDS operation as well, may complete out of order, and while one is pending every wait the compiler inserts
+// becomes a wait for everything in flight.
+// (The cast goes through an integer: a direct generic-to-global pointer cast is a no-op for the optimiser, which
+// folds it away and leaves the generic access.)
+__device__ __forceinline__ uint4 gld16(const void* p) {
+  const u32x4_t v = *(const __attribute__((address_space(1))) u32x4_t*)((unsigned long long)p);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void gst4(void* p, u32 v) {
+  *(__attribute__((address_space(1))) u32*)((unsigned long long)p) = v;
+}
 __device__ __forceinline__ void st16(void* p, uint4 v) { *reinterpret_cast<uint4*>(p) = v; }
 
 // 8 bf16 packed in a uint4 -> 8 floats
