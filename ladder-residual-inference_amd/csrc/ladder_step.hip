@@ -53,10 +53,13 @@
 // small per-launch table: that is what lets the compiler place exact wait counts (vmcnt(8))
 // instead of draining the pipeline.  Weight loads carry the non-temporal hint: each byte is used
 // once per step and must not push the exchanged words out of the caches.  The multiply is
-// v_dot2_f32_bf16 on packed bf16 pairs.  GEMV
-// rows are dealt to workgroups round-robin so that the CUs working at the same time read
-// neighbouring rows (HBM-channel friendly); inside a workgroup the waves split K, partial sums
-// meet in LDS in a fixed order -- no float atomics, bit-reproducible.  Workgroup barriers wait for
+// v_dot2_f32_bf16 on packed bf16 pairs.  Every workgroup owns a run of CONSECUTIVE rows of a matrix,
+// so the eight rows a wave requests together lie one row length (16 KiB in the 70B rank shard) apart.
+// Dealt round-robin (row = workgroup + 256 j) they lie 4 MiB apart, which puts all of a workgroup's
+// requests in flight on the same few DRAM banks: a CU then streams at most about 36 GB/s whatever it
+// has queued, and the workgroup that is served slowest ends every phase 3 to 4 us after the others
+// (measured: 3.13 ms per token round-robin, 3.00 ms consecutive).  Inside a workgroup the waves split K,
+// partial sums meet in LDS in a fixed order -- no float atomics, bit-reproducible.  Workgroup barriers wait for
 // LDS only (wg_sync): __syncthreads() would also wait for the prefetched units.
 //
 // A wave issues at most one instruction every four cycles, so bookkeeping is kept off the layer
@@ -364,14 +367,15 @@ __device__ __forceinline__ float half_row_sum8(float r) {  // every lane of an 8
   r += dpp_mov<0x141>(r);  // row_half_mirror
   return r;
 }
-// sum over the 64 lanes without the LDS crossbar: DPP inside the 16-lane rows, the four row totals through scalar registers
-__device__ __forceinline__ float wave_sum_fast(float v) {
-  const float r = row_sum16(v);
-  const float a = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(r), 0));
-  const float b = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(r), 16));
-  const float c = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(r), 32));
-  const float d = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(r), 48));
-  return (a + b) + (c + d);
+__device__ __forceinline__ float wave_sum_xbar(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, LR_WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max_xbar(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, LR_WAVE));
+  return v;
 }
 __device__ __forceinline__ void reduce8(float* v, float& z0, float& z1) {
   float w[4];
@@ -387,8 +391,8 @@ __device__ __forceinline__ void reduce8(float* v, float& z0, float& z1) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// GEMV work of one workgroup in one matrix ("job").  Items (rows, or up/gate row pairs) are dealt
-// round-robin over the `nwg` participating workgroups: participant w owns items w, w + nwg, ...
+// GEMV work of one workgroup in one matrix ("job").  Items (rows, or up/gate row pairs) are dealt in
+// runs over the participating workgroups: participant w owns items first .. first + n - 1.
 // Its rows are reduced in rounds of NJMAX; inside a round wave (rg, kg) owns rows j = rg (mod nrg)
 // and K-slices kk = kg (mod nkg), RB rows x one 512-element slice per unit.
 // ------------------------------------------------------------------------------------------------
@@ -411,8 +415,8 @@ enum { JK_QKV = 0, JK_W1_SPLIT, JK_WO, JK_W2, JK_HEAD, JK_W1_ALL, JK_NONE, JK_CO
 
 struct Job {  // wave-uniform
   int K2;                  // bytes per row
-  int pair_off, rsh;       // item -> rows: row = w + nwg * (jj >> rsh) + (jj & rsh) * pair_off   (rsh 0 or 1)
-  int w, nwg;              // this workgroup's rank among the participants
+  int pair_off, rsh;       // item -> rows: row = first + (jj >> rsh) + (jj & rsh) * pair_off   (rsh 0 or 1)
+  int rank, first;         // this workgroup's rank among the participants; its first item
   int nj;                  // rows this workgroup owns
   int ksteps, nkg, nrg;    // 512-element K slices; waves along K; waves along rows
   int rg, kg;              // this wave's place
@@ -432,8 +436,11 @@ static_assert(sizeof(Job) == 16 * 4 + 16 + (W8 ? 8 : 0), "16 table words + two p
 __device__ __forceinline__ void build_job(int* rec, int kind, int K, int n_items, int pair_off, int rsh, int w, int nwg,
                                           int wave) {
   Job j;
-  j.K = K; j.K2 = K * WBYTES; j.pair_off = pair_off; j.rsh = rsh; j.w = w; j.nwg = nwg;
-  const int nit = (w >= 0 && n_items > w) ? (n_items - w + nwg - 1) / nwg : 0;
+  j.K = K; j.K2 = K * WBYTES; j.pair_off = pair_off; j.rsh = rsh; j.rank = w;
+  // participant w owns a run of consecutive items (the first n_items % nwg participants one more than the others)
+  const int base = n_items / nwg, rem = n_items % nwg;
+  const int nit = (w >= 0 && w < nwg) ? base + (w < rem ? 1 : 0) : 0;
+  j.first = w >= 0 ? w * base + (w < rem ? w : rem) : 0;
   j.nj = nit << rsh;
   j.ksteps = (K + KSTEP - 1) / KSTEP;
   j.nkg = j.ksteps < NW ? j.ksteps : NW;
@@ -481,7 +488,7 @@ __device__ __forceinline__ void build_row_table(const int* table, int* rowtab) {
     int row_j = rg + (b << j->bsh) + (ii << lg);
     row_j = row_j < njb ? row_j : njb - 1;
     row_j = row_j < 0 ? 0 : row_j;
-    const int row = j->w + j->nwg * (row_j >> j->rsh) + (row_j & ((1 << j->rsh) - 1)) * j->pair_off;
+    const int row = j->first + (row_j >> j->rsh) + (row_j & ((1 << j->rsh) - 1)) * j->pair_off;
     rowtab[i] = (int)((unsigned)row * (unsigned)j->K2);
   }
 }
@@ -490,8 +497,8 @@ __device__ __forceinline__ Job load_job(const int* table, int kind, int wave, co
   const int4* r = reinterpret_cast<const int4*>(table + (kind * NW + wave) * 16);
   const int4 a = r[0], b = r[1], c = r[2], d = r[3];
   Job j;
-  j.K2 = LR_UNI(a.x); j.pair_off = LR_UNI(a.y); j.rsh = LR_UNI(a.z); j.w = LR_UNI(a.w);
-  j.nwg = LR_UNI(b.x); j.nj = LR_UNI(b.y); j.ksteps = LR_UNI(b.z); j.nkg = LR_UNI(b.w);
+  j.K2 = LR_UNI(a.x); j.pair_off = LR_UNI(a.y); j.rsh = LR_UNI(a.z); j.rank = LR_UNI(a.w);
+  j.first = LR_UNI(b.x); j.nj = LR_UNI(b.y); j.ksteps = LR_UNI(b.z); j.nkg = LR_UNI(b.w);
   j.nrg = LR_UNI(c.x); j.rg = LR_UNI(c.y); j.kg = LR_UNI(c.z); j.nk = LR_UNI(c.w);
   j.bsh = LR_UNI(d.x); j.active = LR_UNI(d.y); j.K = LR_UNI(d.z); j.kind = kind;
   j.W = W;
@@ -534,7 +541,7 @@ __device__ __forceinline__ void load_unit(const Job& job, int j0, int jb, int kk
       int j = jb + i * job.nrg;
       j = j < njb ? j : njb - 1;
       const int jj = j0 + j;
-      const int row = job.w + job.nwg * (jj >> job.rsh) + (jj & rmask) * job.pair_off;
+      const int row = job.first + (jj >> job.rsh) + (jj & rmask) * job.pair_off;
       so[i] = (int)((unsigned)row * (unsigned)job.K2);
     }
   }
@@ -733,7 +740,7 @@ __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, con
     // round's units have been multiplied
     float sc0 = 1.0f, sc1 = 1.0f;
     if (tid < (njb >> job.rsh) * M) {
-      const int it_s = job.w + job.nwg * ((j0 >> job.rsh) + tid / M);
+      const int it_s = job.first + (j0 >> job.rsh) + tid / M;
       sc0 = bf_to_f(job.S[it_s]);
       if (EPI == EPI_SWIGLU) sc1 = bf_to_f(job.S[it_s + job.pair_off]);
     }
@@ -776,7 +783,7 @@ __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, con
       s0 = round_bf(s0 * sc0);
       s1 = round_bf(s1 * sc1);
 #endif
-      const int it = job.w + job.nwg * ((j0 >> job.rsh) + jl);
+      const int it = job.first + (j0 >> job.rsh) + jl;
       if (m < p.B) {
         if (EPI == EPI_STORE) coh.st(out_wo + (unsigned)(m * ldo + it), s0, tag);
         if (EPI == EPI_SWIGLU) coh.st(out_wo + (unsigned)(m * ldo + it), swiglu_bf(s0, s1), tag);
@@ -912,7 +919,7 @@ __device__ __forceinline__ void residual_step(const StepParams& p, const Coh& co
   if (stamp && tid == 0) stamp[15] = wall_clock64();
   if (gain == nullptr) return;  // uniform: only the residual was wanted (each lane revisits its own elements later)
 #pragma unroll
-  for (int m = 0; m < M; ++m) ss[m] = wave_sum_fast(ss[m]);
+  for (int m = 0; m < M; ++m) ss[m] = wave_sum(ss[m]);
   if ((tid & 63) == 0) {
 #pragma unroll
     for (int m = 0; m < M; ++m) red[(tid >> 6) * M + m] = ss[m];
@@ -1104,14 +1111,14 @@ __device__ __forceinline__ void attention_compute(const StepParams& p, const Coh
   for (int g = wave; g < G; g += NW) {
     float m = -INFINITY;
     for (int i = lane; i < n; i += 64) m = fmaxf(m, sc[g * sc_ld + i]);
-    m = wave_max(m);
+    m = wave_max_xbar(m);
     float l = 0.0f;
     for (int i = lane; i < n; i += 64) {
       const float e = expf(sc[g * sc_ld + i] - m);
       sc[g * sc_ld + i] = e;
       l += e;
     }
-    l = wave_sum(l);
+    l = wave_sum_xbar(l);
     if (lane == 0) { s_m[g] = m; s_l[g] = l; }
   }
   wg_sync();
@@ -1205,9 +1212,9 @@ __device__ __forceinline__ void attention_merge_slice(const StepParams& p, const
   for (int bh = bh0 + wave; bh <= bh1; bh += NW) {
     float m = -INFINITY, l = 0.0f;
     if (lane < NA) f32x2_from(coh.poll4(p.omlpart + (unsigned)((bh * NA + lane) * 4), tag), m, l);
-    const float mx = wave_max(m);
+    const float mx = wave_max_xbar(m);
     const float w = m == -INFINITY ? 0.0f : expf(m - mx);
-    const float L = wave_sum(w * l);
+    const float L = wave_sum_xbar(w * l);
     if (lane < NA) wbuf[bh * NA_MAX + lane] = L > 0.0f ? w / L : 0.0f;
   }
   wg_sync();

@@ -60,15 +60,29 @@ __device__ __forceinline__ uint4 pack8(const float* f) {
   return v;
 }
 
+// Reductions over the 64 lanes of a wave, every lane getting the result.  Call them with all lanes active.
+// The 16-lane rows are folded with DPP rotations (vector ALU, no LDS crossbar: a __shfl_xor is a ds_bpermute with
+// the latency of an LDS access, six of them in a row for one sum), the four row results meet through scalar registers.
+template <int CTRL>
+__device__ __forceinline__ float lr_dpp(float v) {
+  return __uint_as_float(__builtin_amdgcn_update_dpp(__float_as_uint(v), __float_as_uint(v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float lr_lane(float v, int lane) {
+  return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), lane));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, LR_WAVE);
-  return v;
+  v += lr_dpp<0x128>(v);  // row_ror:8
+  v += lr_dpp<0x124>(v);  // row_ror:4
+  v += lr_dpp<0x4e>(v);   // quad_perm [2,3,0,1]
+  v += lr_dpp<0xb1>(v);   // quad_perm [1,0,3,2]
+  return (lr_lane(v, 0) + lr_lane(v, 16)) + (lr_lane(v, 32) + lr_lane(v, 48));
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, LR_WAVE));
-  return v;
+  v = fmaxf(v, lr_dpp<0x128>(v));
+  v = fmaxf(v, lr_dpp<0x124>(v));
+  v = fmaxf(v, lr_dpp<0x4e>(v));
+  v = fmaxf(v, lr_dpp<0xb1>(v));
+  return fmaxf(fmaxf(lr_lane(v, 0), lr_lane(v, 16)), fmaxf(lr_lane(v, 32), lr_lane(v, 48)));
 }
 
 // silu in fp32 the way the eager reference evaluates it: x / (1 + exp(-x)), rounded to bf16, then
