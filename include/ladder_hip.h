@@ -16,6 +16,11 @@
  *     a hipGraph by stream capture;
  *   - positions are read on the DEVICE from `pos` (int32), never from the host, so a captured
  *     decode step can be replayed after the position buffer has been advanced on the device;
+ *   - what the library remembers between calls are facts about a device (the number of its compute
+ *     units, which kernels have had their dynamic-LDS limit raised, how many workgroups of a kernel
+ *     it can hold, the address of the built-in scratch array of lr_attn_decode_static), looked up once
+ *     per device and kept in atomics: calls from several host threads and for several devices may
+ *     overlap; everything else lives in the caller's buffers;
  *   - the return value is LR_OK or a negative LR_E_* code; on error nothing was launched;
  *   - arithmetic: bf16 storage, fp32 accumulation, one round-to-nearest-even at each point where
  *     the eager reference materialises a bf16 tensor.
@@ -233,6 +238,15 @@ int lr_rope_kv_write(void* qkv, int64_t ldqkv, const void* table, int table_is_g
                      void* k_cache, void* v_cache, int B, int S, int Hq, int Hkv, int hd, int Smax, int block_size,
                      int32_t* err, lr_stream_t stream);
 
+/* KVCache.update (utils.py:50-59):  k_cache[b, h, pos[s], :] = k_val[b, h, s, :], likewise v, for b < B, h < H,
+ * s < S.  k_val / v_val are [B, H, S, hd] views with element strides (stride_b, stride_h, stride_s) and a dense
+ * head dimension; the caches are dense [*, H, Smax, hd].  Positions are read on the device; one outside
+ * [0, Smax) writes nothing for that position and sets *err = LR_DEV_POS_RANGE (err may be NULL), where the
+ * reference's indexed assignment would raise. */
+int lr_kv_update(const void* k_val, const void* v_val, int64_t stride_b, int64_t stride_h, int64_t stride_s,
+                 const int32_t* pos, void* k_cache, void* v_cache, int B, int H, int S, int hd, int Smax, int32_t* err,
+                 lr_stream_t stream);
+
 /* Bytes of fp32 scratch lr_attn_decode needs for (B, Hq, hd, Smax). */
 size_t lr_attn_decode_scratch_bytes(int B, int Hq, int hd, int Smax);
 
@@ -338,6 +352,13 @@ int lr_ladder_decode_step(const lr_ladder_model_t* model, int batch, const int32
                           int64_t ldl, int32_t* next_token, int advance, int32_t* cur_token, int32_t* history,
                           int64_t ld_hist, int hist_len, int pos0, void* workspace, size_t bytes, lr_stream_t stream);
 size_t lr_ladder_step_fail_offset(void);
+
+/* How many workgroups of the step kernel the current device can hold at the same time for this descriptor
+ * and batch (0: shape not supported, or the runtime cannot tell).  The step launches one workgroup per
+ * compute unit and they wait for each other, so lr_ladder_decode_step returns LR_E_LAUNCH unless this is
+ * at least the number of compute units.  No counterpart in the reference (its kernels come from a tracing
+ * compiler and never wait across workgroups); for callers that want to know before they capture a graph. */
+int lr_ladder_step_resident_workgroups(const lr_ladder_model_t* model, int batch);
 
 /* The same step for a weight-only quantised model (every projection of the blocks and the lm_head; the size
  * accounting of gpt_ladder_TP.py:232-237 is the reference's hook for such layers, it ships no quantised layer):

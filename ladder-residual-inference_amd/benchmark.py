@@ -450,6 +450,8 @@ def build_parser():
     p.add_argument("--seed", type=int, default=None, help="seed for weights and prompt")
     p.add_argument("--virtual_tp", type=int, default=None, help="build layers as one rank of this many")
     p.add_argument("--tp_rank", type=int, default=0)
+    p.add_argument("--shard_vocab", action="store_true",
+                   help="with --virtual_tp: the lm_head keeps vocab_size / virtual_tp rows as well")
     p.add_argument("--last_logits_only", action="store_true", help="prefill computes logits of the last position only")
     p.add_argument("--warmup", type=int, default=5)
     p.add_argument("--json", type=Path, default=None, help="write the summary here")
@@ -460,8 +462,10 @@ if __name__ == "__main__":
     args = build_parser().parse_args()
     if args.cuda_graph:
         assert not args.compile
+    if args.shard_vocab and not args.virtual_tp:
+        raise SystemExit("--shard_vocab needs --virtual_tp")
     if args.virtual_tp:
-        set_virtual_tp(args.virtual_tp, args.tp_rank)
+        set_virtual_tp(args.virtual_tp, args.tp_rank, args.shard_vocab)
     print_rank_0(f"flash_kv_decode is set to {args.use_flash_attention}")
     with set_flash_attention(args.use_flash_attention):
         main(args.model_name, args.prompt_length, args.num_samples, args.max_new_tokens, args.batch_size, args.top_k,

@@ -43,11 +43,8 @@ static int launch_decode(const u16* q, int64_t ldq, const u16* kc, const u16* vc
   float* o_part = scratch;
   float* ml_part = scratch + (size_t)B * Hq * nsplit * HD;
   const size_t lds = (size_t)attn_item_lds_floats<HD, G>(chunk_max) * sizeof(float);
-  if (lds > 64 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_attn_decode_partial<HD, G>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return LR_E_LAUNCH;
-  }
+  static std::atomic<unsigned long long> lds_raised{0};
+  if (!lr_raise_lds_limit(reinterpret_cast<const void*>(&k_attn_decode_partial<HD, G>), lds, lds_raised)) return LR_E_LAUNCH;
   k_attn_decode_partial<HD, G><<<dim3(nsplit, Hkv, B), dim3(256), lds, s>>>(q, ldq, kc, vc, pos, o_part, ml_part, Hkv,
                                                                             Smax, nsplit, chunk_max);
   k_attn_decode_combine<HD><<<dim3(Hq, B), dim3(HD), 0, s>>>(o_part, ml_part, y, ldy, Hq, nsplit);
@@ -86,7 +83,6 @@ extern "C" int lr_attn_decode(const void* q, int64_t ldq, const void* k_cache, c
 // up once per device with hipGetSymbolAddress (every device holds its own copy of the array at
 // its own address) and kept in g_static_scratch; host code never passes `scratch` itself.
 constexpr size_t LR_STATIC_SCRATCH_BYTES = LR_ATTN_DECODE_STATIC_MAX_BYTES;
-constexpr int LR_MAX_DEVICES = 64;
 static __device__ __align__(256) unsigned char scratch[LR_STATIC_SCRATCH_BYTES];
 static std::atomic<float*> g_static_scratch[LR_MAX_DEVICES];
 

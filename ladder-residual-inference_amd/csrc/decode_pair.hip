@@ -56,11 +56,8 @@ static int launch_pair_as(const AttnItems& a, const Proj& p, int M, u16* y, int6
   const size_t lds_att = (size_t)attn_item_lds_floats<HD, G>(a.chunk_max) * sizeof(float);
   const size_t lds_band = stream_band_lds_bytes<PAIR_MT, PAIR_UNITS, W8, XL>();
   const size_t lds = lds_att > lds_band ? lds_att : lds_band;
-  if (lds > 64 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_attn_beside_band<HD, G, W8, XL>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return LR_E_LAUNCH;
-  }
+  static std::atomic<unsigned long long> lds_raised{0};
+  if (!lr_raise_lds_limit(reinterpret_cast<const void*>(&k_attn_beside_band<HD, G, W8, XL>), lds, lds_raised)) return LR_E_LAUNCH;
   k_attn_beside_band<HD, G, W8, XL><<<dim3((unsigned)(a.n_items + p.nwg)), dim3(256), lds, s>>>(a, p, M);
   k_attn_decode_combine<HD><<<dim3(Hq, B), dim3(HD), 0, s>>>(a.o_part, a.ml_part, y, ldy, Hq, a.nsplit);
   return lr_launch_status();
@@ -69,7 +66,7 @@ static int launch_pair_as(const AttnItems& a, const Proj& p, int M, u16* y, int6
 // (the band's inputs in whole lines or in fragment layout: the choice lr_linear_multi makes for the same rows)
 template <int HD, int G, bool W8>
 static int launch_pair(const AttnItems& a, const Proj& p, int M, u16* y, int64_t ldy, int B, hipStream_t s) {
-  if (!W8 && M >= LR_SG_XLDS_M16_FROM) return launch_pair_as<HD, G, false, true>(a, p, M, y, ldy, B, s);
+  if (!W8 && M >= XLDS_M16_FROM) return launch_pair_as<HD, G, false, true>(a, p, M, y, ldy, B, s);
   return launch_pair_as<HD, G, W8, false>(a, p, M, y, ldy, B, s);
 }
 
@@ -111,7 +108,7 @@ static int beside(const void* q, int64_t ldq, const void* k_cache, const void* v
   if ((int64_t)a.nsplit * a.Hkv * B > 0x3fffffff) return LR_E_UNSUPPORTED;
   a.n_items = a.nsplit * a.Hkv * B;
   if (!((hd == 128 || hd == 64) && (G == 1 || G == 2 || G == 4 || G == 8))) return LR_E_UNSUPPORTED;
-  const int ncu = sb_num_cus();
+  const int ncu = lr_num_cus();
   if (ncu < 1) return LR_E_LAUNCH;
   plan(p, M, p.pair_off ? 16 : 16 * PAIR_UNITS, ncu);
   hipStream_t s = (hipStream_t)stream;

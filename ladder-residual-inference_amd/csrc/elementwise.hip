@@ -344,6 +344,43 @@ extern "C" int lr_rope_kv_write(void* qkv, int64_t ldqkv, const void* table, int
   return lr_launch_status();
 }
 
+// ------------------------------------------------------------------------------------ KVCache.update
+// k_cache[b, h, pos[s], :] = k_val[b, h, s, :] (and v), one workgroup per (b, h, s); the values may be a strided view
+// (element strides for b, h, s; the head dimension is dense).  Positions come from the device, as everywhere.
+__global__ __launch_bounds__(64) void k_kv_update(const u16* __restrict__ kval, const u16* __restrict__ vval,
+                                                  int64_t sb, int64_t sh, int64_t ss, const int32_t* __restrict__ pos,
+                                                  u16* __restrict__ kc, u16* __restrict__ vc, int H, int S, int hd,
+                                                  int Smax, int32_t* err) {
+  const int s_ = blockIdx.x % S, h = (blockIdx.x / S) % H, b = blockIdx.x / (S * H);
+  const int at = pos[s_];
+  if (at < 0 || at >= Smax) {
+    if (err && threadIdx.x == 0) *err = LR_DEV_POS_RANGE;
+    return;
+  }
+  const int64_t src = (int64_t)b * sb + (int64_t)h * sh + (int64_t)s_ * ss;
+  const int64_t dst = (((int64_t)b * H + h) * Smax + at) * hd;
+  for (int c = threadIdx.x * 8; c < hd; c += 64 * 8) {
+    st16(kc + dst + c, ld16(kval + src + c));
+    st16(vc + dst + c, ld16(vval + src + c));
+  }
+}
+
+extern "C" int lr_kv_update(const void* k_val, const void* v_val, int64_t stride_b, int64_t stride_h, int64_t stride_s,
+                            const int32_t* pos, void* k_cache, void* v_cache, int B, int H, int S, int hd, int Smax,
+                            int32_t* err, lr_stream_t stream) {
+  LR_REQUIRE_PTR(k_val);
+  LR_REQUIRE_PTR(v_val);
+  LR_REQUIRE_PTR(k_cache);
+  LR_REQUIRE_PTR(v_cache);
+  if (pos == nullptr) return LR_E_NULL;
+  if (B <= 0 || H <= 0 || S <= 0 || hd <= 0 || Smax <= 0 || (int64_t)B * H * S > 0x7fffffff) return LR_E_SHAPE;
+  if (hd % 8 || stride_b % 8 || stride_h % 8 || stride_s % 8) return LR_E_ALIGN;
+  k_kv_update<<<dim3((unsigned)(B * H * S)), dim3(64), 0, (hipStream_t)stream>>>(
+      (const u16*)k_val, (const u16*)v_val, stride_b, stride_h, stride_s, pos, (u16*)k_cache, (u16*)v_cache, H, S, hd,
+      Smax, err);
+  return lr_launch_status();
+}
+
 // ------------------------------------------------------------------------------------ argmax
 // One workgroup of 1024 lanes per row.  (value, index) pairs are merged with "greater value, or
 // equal value and lower index", which makes the result independent of the merge order.

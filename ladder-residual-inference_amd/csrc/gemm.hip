@@ -340,13 +340,8 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
 static int launch_gemm_big(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
                            int pair_off, hipStream_t s) {
   constexpr size_t lds = (size_t)2 * (GM + GN) * LDT * sizeof(u16);
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_big), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds) != hipSuccess)
-      return LR_E_LAUNCH;
-    attr_set = true;
-  }
+  static std::atomic<unsigned long long> lds_raised{0};
+  if (!lr_raise_lds_limit(reinterpret_cast<const void*>(&k_gemm_big), lds, lds_raised)) return LR_E_LAUNCH;
   const int gn = pair_off ? GN / 2 : GN;
   const int tm = (M + GM - 1) / GM, tn = (N + gn - 1) / gn;
   k_gemm_big<<<dim3((unsigned)(tm * tn)), dim3(256), lds, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy, M, N, K,

@@ -1510,17 +1510,6 @@ struct Layout {
   size_t ctrl, abuf, mbuf, qkv, act, opart, mlpart, cand, y, total;
 };
 
-static int num_cus() {
-  static int n = 0;
-  if (n == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0;
-    n = prop.multiProcessorCount;
-  }
-  return n;
-}
-
 // keys one attention workgroup can hold in registers: the V groups (ATT_NI * NW * keys per wave)
 // and the K tiles of the score pass (ATT_KT * NW * 32) both have to cover its key range
 static int att_capacity(int hd) {
@@ -1653,28 +1642,53 @@ static int validate(const lr_ladder_model_t* md, int B) {
     if (most >= 0x7fffffff || (int64_t)md->dim * md->ffn >= 0x7fffffff) return LR_E_UNSUPPORTED;
   }
   if (lds_need(B, md->head_dim, G, md->dim, md->ffn, md->n_head) > 160 * 1024) return LR_E_UNSUPPORTED;
-  const int nwg = num_cus();
+  const int nwg = lr_num_cus();
   if (nwg < 2) return LR_E_LAUNCH;
   if (md->dim > NJMAX * nwg) return LR_E_UNSUPPORTED;  // a workgroup's rows of wo / w2 fit one reduction round
+  // Overwriting an exchange array is ordered by data flow through the rows every workgroup produces (see the layer
+  // loop): a workgroup without a row of wqkv, or a weight-streaming workgroup without a row pair of w1, would not
+  // be part of that chain.  Such shapes (fewer q/k/v rows than CUs) are left to the per-op kernels.
+  if ((md->n_head + 2 * md->n_kv_head) * md->head_dim < nwg) return LR_E_UNSUPPORTED;
   const AttSplit as = pick_split(md, nwg);
   if (as.nak > NA_MAX || (md->smax + as.nak - 1) / as.nak > att_capacity(md->head_dim) || as.nak * as.nah >= nwg ||
       md->n_kv_head % as.nah)
     return LR_E_UNSUPPORTED;
+  if (md->ffn < nwg - as.nak * as.nah) return LR_E_UNSUPPORTED;
   if (!md->tok_embeddings || !md->norm || !md->output || !md->freqs_cis || !md->layers_dev) return LR_E_NULL;
   return LR_OK;
+}
+
+// Workgroups of one instance that can be resident on the current device at once, for `lds` bytes of dynamic LDS
+// (occupancy per CU x CUs; 0 if the runtime cannot tell).  The answer for the largest size asked so far is kept per
+// device: occupancy does not grow with the LDS size, so a smaller request is covered by it.
+template <int M, int HD, int G>
+static int resident_workgroups(size_t lds) {
+  static std::atomic<unsigned long long> lds_raised{0};
+  static std::atomic<size_t> asked[LR_MAX_DEVICES];
+  static std::atomic<int> fits[LR_MAX_DEVICES];
+  const void* fn = reinterpret_cast<const void*>(&k_ladder_step<M, HD, G>);
+  const int dev = lr_current_device();
+  if (dev < 0 || !lr_raise_lds_limit(fn, lds, lds_raised)) return 0;
+  if (lds <= asked[dev].load(std::memory_order_acquire)) return fits[dev].load(std::memory_order_relaxed);
+  int per_cu = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, NT, lds) != hipSuccess || per_cu < 0) return 0;
+  const int n = per_cu * lr_num_cus();
+  if (n > 0) {  // (a size that does not fit is asked about again next time: nothing to remember)
+    fits[dev].store(n, std::memory_order_relaxed);
+    asked[dev].store(lds, std::memory_order_release);
+  }
+  return n;
 }
 
 template <int M, int HD, int G>
 static int launch_step(const StepParams& sp, int Hq, hipStream_t s) {
   const size_t lds = lds_bytes<M, HD, G>(sp.D, sp.I, Hq);
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_ladder_step<M, HD, G>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
-      return LR_E_LAUNCH;
-    attr_set = true;
-  }
-  k_ladder_step<M, HD, G><<<dim3(num_cus()), dim3(NT), lds, s>>>(sp);
+  // Every workgroup polls words that the others write, so all of them have to be resident at the same time: a
+  // launch that the device cannot hold whole is refused here instead of running into its bounded waits.  (What
+  // else occupies the device at that moment is not known here; that case ends in LR_DEV_WAIT_EXPIRED.)
+  const int grid = lr_num_cus();
+  if (resident_workgroups<M, HD, G>(lds) < grid) return LR_E_LAUNCH;
+  k_ladder_step<M, HD, G><<<dim3(grid), dim3(NT), lds, s>>>(sp);
   return lr_launch_status();
 }
 
@@ -1692,17 +1706,28 @@ int g_prof_t0 = 0;
 extern "C" size_t lr_ladder_step_profile(void* device_buffer, int first_slot) {
   g_prof = reinterpret_cast<unsigned long long*>(device_buffer);
   g_prof_t0 = first_slot;
-  return (size_t)num_cus() * PROF_SLOTS * PROF_POINTS * sizeof(unsigned long long);
+  return (size_t)lr_num_cus() * PROF_SLOTS * PROF_POINTS * sizeof(unsigned long long);
 }
 #endif
 
 #if !LR_STEP_W8
 extern "C" size_t lr_ladder_step_workspace_bytes(const lr_ladder_model_t* md, int batch) {
   if (validate(md, batch) != LR_OK) return 0;
-  return make_layout(md, batch, num_cus()).total;
+  return make_layout(md, batch, lr_num_cus()).total;
 }
 
 extern "C" size_t lr_ladder_step_fail_offset(void) { return offsetof(Ctrl, fail); }
+
+extern "C" int lr_ladder_step_resident_workgroups(const lr_ladder_model_t* md, int batch) {
+  if (validate(md, batch) != LR_OK) return 0;
+  const int G = md->n_head / md->n_kv_head, hd = md->head_dim;
+#define LR_RES(MV, HDV, GV) \
+  if (batch == MV && hd == HDV && G == GV) \
+    return resident_workgroups<MV, HDV, GV>(lds_bytes<MV, HDV, GV>(md->dim, md->ffn, md->n_head));
+  LR_STEP_INSTANCES(LR_RES)
+#undef LR_RES
+  return 0;
+}
 
 extern "C" int lr_ladder_step_init(const lr_ladder_model_t* md, int batch, void* workspace, size_t bytes,
                                    lr_stream_t stream) {
@@ -1710,9 +1735,9 @@ extern "C" int lr_ladder_step_init(const lr_ladder_model_t* md, int batch, void*
   if (rc != LR_OK) return rc;
   LR_REQUIRE_PTR(workspace);
   if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return LR_E_ALIGN;
-  const Layout l = make_layout(md, batch, num_cus());
+  const Layout l = make_layout(md, batch, lr_num_cus());
   if (bytes < l.total) return LR_E_SHAPE;
-  k_step_init<<<dim3(64), dim3(256), 0, (hipStream_t)stream>>>(reinterpret_cast<Ctrl*>(workspace), (unsigned)num_cus(),
+  k_step_init<<<dim3(64), dim3(256), 0, (hipStream_t)stream>>>(reinterpret_cast<Ctrl*>(workspace), (unsigned)lr_num_cus(),
                                                               reinterpret_cast<unsigned*>(workspace),
                                                               (unsigned)(l.total / 4));
   return lr_launch_status();
@@ -1734,7 +1759,7 @@ extern "C" int LR_STEP_ENTRY(const lr_ladder_model_t* md, int batch, const int32
   LR_REQUIRE_PTR(logits);
   if (tokens == nullptr || pos == nullptr) return LR_E_NULL;
   if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return LR_E_ALIGN;
-  const int nwg = num_cus();
+  const int nwg = lr_num_cus();
   const Layout l = make_layout(md, batch, nwg);
   if (bytes < l.total || ldl < md->out_rows || l.total > 0x7fffffffu) return LR_E_SHAPE;
   if (history && (ld_hist < hist_len || hist_len <= 0)) return LR_E_SHAPE;

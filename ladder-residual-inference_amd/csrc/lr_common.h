@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/ladder_hip.h"
 
 #define LR_WAVE 64
@@ -105,3 +107,40 @@ static inline bool lr_misaligned(const void* p) { return (reinterpret_cast<uintp
   } while (0)
 
 static inline int lr_launch_status() { return hipGetLastError() == hipSuccess ? LR_OK : LR_E_LAUNCH; }
+
+// ---- what the library remembers between calls: facts about a device, looked up once per DEVICE, in atomics (calls
+//      from several host threads and on several devices may overlap; two first calls store the same value).
+constexpr int LR_MAX_DEVICES = 64;
+
+static inline int lr_current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= LR_MAX_DEVICES) return -1;
+  return dev;
+}
+
+// compute units of the current device (0: no device)
+static inline int lr_num_cus() {
+  static std::atomic<int> n[LR_MAX_DEVICES];
+  const int dev = lr_current_device();
+  if (dev < 0) return 0;
+  int v = n[dev].load(std::memory_order_relaxed);
+  if (v == 0) {
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) return 0;
+    n[dev].store(v, std::memory_order_relaxed);
+  }
+  return v;
+}
+
+// A kernel that needs more than 64 KiB of dynamic LDS has its limit raised once per device.  `done` is a per-kernel
+// word (one bit per device) owned by the caller; returns false if the runtime refuses.
+static inline bool lr_raise_lds_limit(const void* kernel, size_t bytes, std::atomic<unsigned long long>& done) {
+  if (bytes <= 64 * 1024) return true;
+  const int dev = lr_current_device();
+  if (dev < 0) return false;
+  const unsigned long long bit = 1ull << dev;
+  if (done.load(std::memory_order_acquire) & bit) return true;
+  // the limit is set to all of the CU's LDS: a later call of the same kernel with another size needs no second visit
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess) return false;
+  done.fetch_or(bit, std::memory_order_release);
+  return true;
+}

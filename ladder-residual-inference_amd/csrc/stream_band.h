@@ -15,15 +15,9 @@ constexpr int OOB = (int)0x80000000;  // a buffer offset beyond every resource: 
 // always with the 32- and 64-row bands; the 16-row band has both forms and the launcher picks by the row count
 // (70B rank shard, ms per step, fragment layout / whole lines: 4 rows 4.99 / 5.12, 8 rows 5.14 / 5.19, 16 rows
 // 6.26 / 6.00; 8B, 16 rows: 4.00 / 3.78)
-#ifndef LR_SG_XLDS_MIN
-#define LR_SG_XLDS_MIN 32
-#endif
-#ifndef LR_SG_XLDS_M16_FROM
-#define LR_SG_XLDS_M16_FROM 9
-#endif
-#ifndef LR_SG_W_AUX
-#define LR_SG_W_AUX 2          // weights: non-temporal (every line is used exactly once)
-#endif
+constexpr int XLDS_MIN_MT = 32;       // band heights that always read their inputs in whole lines
+constexpr int XLDS_M16_FROM = 9;      // input rows from which the 16-row band does too
+constexpr int AUX_WEIGHTS = 2;        // weights: non-temporal (every line is used exactly once)
 
 struct Proj {
   const u16* x;
@@ -50,7 +44,7 @@ __device__ __forceinline__ u32 sb_fp8_pair(u32 v) {
   return __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v, 1.0f, HI));
 }
 
-template <int MT, int UNITS, bool W8 = false, bool XL = (MT >= LR_SG_XLDS_MIN)>
+template <int MT, int UNITS, bool W8 = false, bool XL = (MT >= XLDS_MIN_MT)>
 constexpr size_t stream_band_lds_bytes() {
   constexpr int LRW = (W8 ? 2 * KC : KC) + 8;
   return (size_t)NWV * (UNITS * 16 * LRW + (XL ? MT * LRW : 0)) * sizeof(u16);
@@ -61,18 +55,15 @@ constexpr size_t stream_band_lds_bytes() {
 // 256 bytes, now 256 elements of K, which are expanded to bf16 (exactly: e4m3 is a subset of bf16) on their way
 // into the LDS piece; the sum is rounded to bf16, multiplied by the row's scale and rounded again, as
 // F.linear(x, w.to(bf16)) * scales does, before the epilogue sees it.
-template <int MT, int UNITS, bool W8 = false, bool XL = (MT >= LR_SG_XLDS_MIN)>
+template <int MT, int UNITS, bool W8 = false, bool XL = (MT >= XLDS_MIN_MT)>
 __device__ __forceinline__ void stream_band(const Proj& p, const int M, const int band, u16* sg_smem) {
   static_assert(!W8 || MT == 16, "the e4m3 path is built for up to 16 input rows");
   constexpr int KCW = W8 ? 256 : 128;  // k elements per chunk
   constexpr int LRW = KCW + 8;         // LDS row length in elements
   constexpr int WB = W8 ? 1 : 2;       // bytes per weight
-#ifndef LR_SG_W8_SETS
-#define LR_SG_W8_SETS 2
-#endif
   // weight chunks in flight per wave: the e4m3 variant has twice the A fragments and input registers per chunk
   // and gives up two of its four sets for a second workgroup per CU
-  constexpr int NS = W8 ? LR_SG_W8_SETS : SETS;
+  constexpr int NS = W8 ? 2 : SETS;
   constexpr int MTILES = MT / 16, KS = KCW / 32, NLD = UNITS * 4;
   constexpr int NV = UNITS * MTILES * 4;  // accumulator registers per lane
   // XL: the inputs too are loaded in whole lines (4 rows x 256 bytes per instruction) and take the trip through
@@ -148,7 +139,7 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
     const bool kok = k0 + l16 * (16 / WB) < K;
 #pragma unroll
     for (int i = 0; i < NLD; ++i)
-      dst[i] = __builtin_amdgcn_raw_buffer_load_b128(wres, (kok && woff[i] != OOB) ? woff[i] : OOB, k0 * WB, LR_SG_W_AUX);
+      dst[i] = __builtin_amdgcn_raw_buffer_load_b128(wres, (kok && woff[i] != OOB) ? woff[i] : OOB, k0 * WB, AUX_WEIGHTS);
   };
   auto issue_x = [&](int ci, u32x4_t (&dst)[MTILES][KS]) {
     const int k0 = (ci * NWV + wave) * KCW;
@@ -333,17 +324,6 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
       yg[(int64_t)m * ldy + n0 + r] = f_to_bf(s0);
     }
   }
-}
-
-static int sb_num_cus() {
-  static int n = 0;
-  if (n == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0;
-    n = prop.multiProcessorCount;
-  }
-  return n;
 }
 
 // Rows per workgroup: the rows are spread evenly over whole rounds of the CUs, at most `cap` per

@@ -32,23 +32,18 @@ __global__ __launch_bounds__(NWV * 64) void k_stream_gemm(const Proj p0, const P
   stream_band<MT, UNITS, W8, XL>(p, M, second ? (int)blockIdx.x - p0.nwg : (int)blockIdx.x, sg_smem);
 }
 
-template <int MT, int UNITS, bool W8 = false, bool XL = (MT >= LR_SG_XLDS_MIN)>
+template <int MT, int UNITS, bool W8 = false, bool XL = (MT >= XLDS_MIN_MT)>
 static int launch_units(Proj& a, Proj& b, int M, hipStream_t s) {
   constexpr size_t lds = stream_band_lds_bytes<MT, UNITS, W8, XL>();
-  static bool attr_set = false;
-  if (!attr_set && lds > 64 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_stream_gemm<MT, UNITS, W8, XL>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return LR_E_LAUNCH;
-    attr_set = true;
-  }
+  static std::atomic<unsigned long long> lds_raised{0};
+  if (!lr_raise_lds_limit(reinterpret_cast<const void*>(&k_stream_gemm<MT, UNITS, W8, XL>), lds, lds_raised)) return LR_E_LAUNCH;
   k_stream_gemm<MT, UNITS, W8, XL><<<dim3((unsigned)(a.nwg + b.nwg)), dim3(NWV * 64), lds, s>>>(a, b, M);
   return LR_OK;
 }
 
 template <int MT>
 static int launch(Proj& a, Proj& b, int M, int units, hipStream_t s) {
-  if (MT == 16 && M >= LR_SG_XLDS_M16_FROM)  // the 16-row band with its inputs read in whole lines
+  if (MT == 16 && M >= XLDS_M16_FROM)  // the 16-row band with its inputs read in whole lines
     return units == 2 ? launch_units<MT, 2, false, true>(a, b, M, s) : launch_units<MT, 1, false, true>(a, b, M, s);
   return units == 2 ? launch_units<MT, 2>(a, b, M, s) : launch_units<MT, 1>(a, b, M, s);
 }
@@ -76,7 +71,7 @@ extern "C" int lr_linear_multi(const lr_projection_t* proj, int n_proj, int M, l
     const int rc = sb_fill_projection(proj[i], pr[i]);
     if (rc != LR_OK) return rc;
   }
-  const int ncu = sb_num_cus();
+  const int ncu = lr_num_cus();
   if (ncu < 1) return LR_E_LAUNCH;
   const int units = pick_units_and_plan(pr, n_proj, M, ncu);
   hipStream_t s = (hipStream_t)stream;
@@ -94,7 +89,7 @@ int stream_fp8_multi(const lr_projection_fp8_t* proj, int n_proj, int M, lr_stre
     const int rc = sb_fill_projection_fp8(proj[i], pr[i]);
     if (rc != LR_OK) return rc;
   }
-  const int ncu = sb_num_cus();
+  const int ncu = lr_num_cus();
   if (ncu < 1) return LR_E_LAUNCH;
   const int units = pick_units_and_plan(pr, n_proj, M, ncu);
   hipStream_t s = (hipStream_t)stream;

@@ -35,6 +35,8 @@ _PROTOS = {
     "lr_swiglu": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_int, c_void_p]),
     "lr_rope_kv_write": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                  c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "lr_kv_update": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                             c_int, c_int, c_int, c_void_p, c_void_p]),
     "lr_attn_decode_scratch_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "lr_attn_decode": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int,
                                c_int, c_int, c_void_p, c_size_t, c_void_p]),
@@ -58,6 +60,7 @@ _PROTOS = {
     "lr_ladder_decode_step_fp8": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int,
                                           c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "lr_ladder_step_fail_offset": (c_size_t, []),
+    "lr_ladder_step_resident_workgroups": (c_int, [c_void_p, c_int]),
 }
 
 
@@ -314,9 +317,12 @@ def linear_fp8(x: torch.Tensor, w8: torch.Tensor, scales: torch.Tensor, out: tor
     need = int(lib.lr_linear_fp8_scratch_bytes(M, N, K))
     scratch = None
     if need:
-        scratch = _FP8_SCRATCH.get(x.device)
+        # one expansion buffer per (device, stream): calls on one stream are ordered and share it; calls on two
+        # streams (a block's attention and MLP chains with overlap_modules) expand different matrices at once
+        key = (x.device, _stream())
+        scratch = _FP8_SCRATCH.get(key)
         if scratch is None or scratch.numel() < need:
-            scratch = _FP8_SCRATCH[x.device] = torch.empty(need, dtype=torch.uint8, device=x.device)
+            scratch = _FP8_SCRATCH[key] = torch.empty(need, dtype=torch.uint8, device=x.device)
     _check(lib.lr_linear_fp8(_dev(x), ldx, w8.data_ptr(), _dev(scales), _dev(out), ldy, M, N, K,
                              None if scratch is None else scratch.data_ptr(), need, _stream()), "lr_linear_fp8")
     return out
@@ -421,6 +427,18 @@ def rope_kv_write(qkv, table, table_is_gathered, pos, k_cache, v_cache, B, S, Hq
                                    _dev(k_cache), _dev(v_cache), B, S, Hq, Hkv, hd, Smax, table.shape[0],
                                    device_error_word(qkv.device).data_ptr(), _stream()),
            "lr_rope_kv_write")
+
+
+def kv_update(k_val, v_val, pos, k_cache, v_cache):
+    """KVCache.update: k_cache[:B, :, pos] = k_val ([B, H, S, hd], any strides with a dense last dimension)."""
+    B, H, S, hd = k_val.shape
+    assert v_val.shape == k_val.shape and v_val.stride() == k_val.stride() and k_val.stride(-1) == 1
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape == v_cache.shape
+    Bmax, Hc, Smax, hdc = k_cache.shape
+    assert B <= Bmax and Hc == H and hdc == hd and pos.dtype == torch.int32 and pos.is_cuda and pos.numel() == S
+    sb, sh, ss, _ = k_val.stride()
+    _check(load().lr_kv_update(_dev(k_val), _dev(v_val), sb, sh, ss, pos.data_ptr(), _dev(k_cache), _dev(v_cache), B, H,
+                               S, hd, Smax, device_error_word(k_val.device).data_ptr(), _stream()), "lr_kv_update")
 
 
 def attn_decode_scratch_bytes(B, Hq, hd, Smax) -> int:
@@ -592,6 +610,12 @@ class FusedLadderStep:
             most = max((d.n_head + 2 * d.n_kv_head) * d.head_dim, 2 * d.ffn, d.out_rows) * d.dim
             self.supported = self.supported and d.dim % 16 == 0 and d.ffn % 16 == 0 and \
                 (d.n_head * d.head_dim) % 16 == 0 and max(most, d.dim * d.ffn) < 0x7fffffff
+        if self.supported:
+            # one workgroup per compute unit, all resident at once: a device that cannot hold them leaves the model
+            # to the per-op kernels (the launch itself would return LR_E_LAUNCH)
+            with torch.cuda.device(dev):
+                self.resident = int(lib.lr_ladder_step_resident_workgroups(ctypes.byref(self.desc), batch))
+            self.supported = self.resident >= torch.cuda.get_device_properties(dev).multi_processor_count
         self.workspace = None
         if self.supported:
             self.workspace = _aligned_bytes(self.bytes, dev)

@@ -3,10 +3,11 @@
 Module tree and public surface follow the reference (gpt_ladder_TP.py:210-288): children
 `tok_embeddings`, `layers`, `norm`, `output`; `setup_caches(max_batch_size, max_seq_length)`;
 `forward(idx [B, S], input_pos [S]) -> logits [B, S, V]`; `from_name`.  forward() is a fixed
-sequence of libladder_hip.so launches over preallocated buffers: no torch kernels, no
-allocation after the first call for a given (B, S), no host synchronisation, positions read from
-the device tensor `input_pos` -- so one decode step can be captured into a hipGraph and replayed
-while `input_pos` and the token buffer are advanced on the device."""
+sequence of libladder_hip.so launches over preallocated buffers: no allocation after the first call
+for a given (B, S), no host synchronisation, positions read from the device tensor `input_pos` --
+so one decode step can be captured into a hipGraph and replayed while `input_pos` and the token
+buffer are advanced on the device.  The only torch kernels are dtype / layout conversions of
+arguments that arrive in another form (int64 positions, a non-contiguous token tensor)."""
 from typing import Dict, Optional
 
 import torch
@@ -36,6 +37,11 @@ class Workspace:
         self.h = e(rows, 2 * cfg.ffn_local)
         self.act = e(rows, cfg.ffn_local)   # activated MLP input where SwiGLU is not fused into the projection
         self.logits = e(B, S if all_logits else 1, cfg.output_rows)
+        if S > 1 and not all_logits:
+            # prefill with the head on the last position only: the B last rows are gathered out of the [B * S, D]
+            # buffers with the row-gather kernel (lr_embed) into these
+            self.last_rows = (torch.arange(1, B + 1, dtype=torch.int32, device=device) * S - 1).contiguous()
+            self.xl, self.d1l, self.d2l, self.xnl = e(B, D), e(B, D), e(B, D), e(B, D)
         self.next_token = torch.empty(B, 1, dtype=torch.int32, device=device)
         self.next_token_valid_for = None   # set by a fused decode step that already chose the token
         self.scratch = None
@@ -145,12 +151,11 @@ class GPTBase(nn.Module):
         final_d1, final_d2 = self._run_layers(ws, pos)
         cfg = self.config
         if self.last_logits_only and S > 1:
-            # only row S-1 of each sequence feeds the head: copy those B rows out, then norm + lm_head
-            last = lambda t: None if t is None else t.view(B, S, -1)[:, S - 1].contiguous()
-            xl = last(ws.x)
-            xn = torch.empty_like(xl)
-            _hip.add_rmsnorm(xl, last(final_d1), last(final_d2), self.norm.weight, None, xn, cfg.norm_eps)
-            _hip.module_linear(xn, self.output, ws.logits.view(B, -1))
+            # only row S-1 of each sequence feeds the head: gather those B rows, then norm + lm_head
+            last = lambda t, out: None if t is None else _hip.embed(t.view(B * S, -1), ws.last_rows, out)
+            _hip.add_rmsnorm(last(ws.x, ws.xl), last(final_d1, ws.d1l), last(final_d2, ws.d2l), self.norm.weight, None,
+                             ws.xnl, cfg.norm_eps)
+            _hip.module_linear(ws.xnl, self.output, ws.logits.view(B, -1))
         else:
             _hip.add_rmsnorm(ws.x, final_d1, final_d2, self.norm.weight, None, ws.xn, cfg.norm_eps)
             _hip.module_linear(ws.xn, self.output, ws.logits.view(B * S, -1))

@@ -47,13 +47,20 @@ def is_hf_state_dict(sd: StateDict) -> bool:
     return any(k.startswith("model.layers.") or k == "model.embed_tokens.weight" for k in sd)
 
 
-def convert_hf_state_dict(sd: StateDict, n_head: int, n_kv_head: int) -> StateDict:
-    """Un-sharded HF Llama(-Ladder) state dict -> un-sharded gpt_fast state dict (fused projections)."""
+def convert_hf_state_dict(sd: StateDict, n_head: int, n_kv_head: int, head_dim: Optional[int] = None) -> StateDict:
+    """HF Llama(-Ladder) state dict -> gpt_fast state dict (fused projections).  n_head / n_kv_head are the head
+    counts of the tensors AS GIVEN: the global ones for an un-sharded checkpoint, the per-rank ones for a slice.
+    With head_dim the q / k row counts are checked against them (a wrong head count would permute rows silently)."""
     out: StateDict = {}
     layers = sorted({int(k.split(".")[2]) for k in sd if k.startswith("model.layers.")})
     out["tok_embeddings.weight"] = sd["model.embed_tokens.weight"]
     for i in layers:
         src, dst = f"model.layers.{i}.", f"layers.{i}."
+        if head_dim is not None:
+            for name, heads in (("q_proj", n_head), ("k_proj", n_kv_head)):
+                rows = sd[src + f"self_attn.{name}.weight"].shape[0]
+                if rows != heads * head_dim:
+                    raise ValueError(f"{src}self_attn.{name}.weight has {rows} rows, expected {heads} heads x {head_dim}")
         q = _interleave_rope_rows(sd[src + "self_attn.q_proj.weight"], n_head)
         k = _interleave_rope_rows(sd[src + "self_attn.k_proj.weight"], n_kv_head)
         v = sd[src + "self_attn.v_proj.weight"]
@@ -86,9 +93,18 @@ def model_args_from_hf_config(cfg: Union[str, dict], **overrides) -> dict:
             raise ValueError(f"rope_scaling of type {kind!r} is not supported (the reference implements llama3 only)")
         kw["rope_scaling"] = {k: scaling[k] for k in ("factor", "low_freq_factor", "high_freq_factor",
                                                       "original_max_position_embeddings")}
+    # configuration_llama_ladder.py:38-45: no field (a plain Llama config.json) or null means NO ladder layer -- every
+    # block dense -- and an int means "the last n layers".  (ModelArgs itself reads None as "all layers", the
+    # gpt_fast convention, so the absent field must not be passed on as None.)
     ladder = cfg.get("ladder_layers")
-    if ladder is not None:   # configuration_llama_ladder.py:38-45: an int means "the last n layers"
-        kw["ladder_layers"] = list(range(n_layer - ladder, n_layer)) if isinstance(ladder, int) else list(ladder)
+    if ladder is None:
+        kw["ladder_layers"] = []
+    elif isinstance(ladder, int):
+        kw["ladder_layers"] = list(range(n_layer - ladder, n_layer))
+    elif isinstance(ladder, list):
+        kw["ladder_layers"] = list(ladder)
+    else:
+        raise ValueError(f"Invalid ladder_layers type: {type(ladder)}")
     kw.update(overrides)
     return kw
 
@@ -165,7 +181,10 @@ def read_state_dict(path: str) -> StateDict:
         from safetensors.torch import load_file
 
         return load_file(path)
-    sd = torch.load(path, map_location="cpu", weights_only=True, mmap=True)
+    try:
+        sd = torch.load(path, map_location="cpu", weights_only=True, mmap=True)
+    except (RuntimeError, ValueError):   # a legacy (non-zip) torch file cannot be memory-mapped
+        sd = torch.load(path, map_location="cpu", weights_only=True)
     return sd.get("model", sd) if isinstance(sd, dict) and "model" in sd and isinstance(sd["model"], dict) else sd
 
 
@@ -177,7 +196,9 @@ def load_checkpoint(model: torch.nn.Module, checkpoint: Union[str, StateDict], a
     cfg = model.config
     sd = read_state_dict(checkpoint) if isinstance(checkpoint, (str, os.PathLike)) else dict(checkpoint)
     if is_hf_state_dict(sd):
-        sd = convert_hf_state_dict(sd, cfg.n_head, cfg.n_local_heads)
+        # an already sharded checkpoint holds this rank's heads only
+        heads = (cfg.n_head_local, cfg.n_kv_local) if already_sharded else (cfg.n_head, cfg.n_local_heads)
+        sd = convert_hf_state_dict(sd, heads[0], heads[1], cfg.head_dim)
     if not already_sharded:
         sd = shard_state_dict(sd, cfg.n_head, cfg.n_local_heads, cfg.head_dim, cfg.tp_world_size, cfg.tp_rank,
                               cfg.shard_vocab)

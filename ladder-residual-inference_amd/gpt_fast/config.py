@@ -40,14 +40,17 @@ class ModelArgs:
     # rank shard: None -> the process-wide virtual setting of gpt_fast.tp
     tp_world_size: Optional[int] = None
     tp_rank: Optional[int] = None
-    # lm_head keeps vocab_size // tp_world_size rows (the reference replicates the full head)
-    shard_vocab: bool = False
+    # lm_head keeps vocab_size // tp_world_size rows (the reference replicates the full head); None -> the
+    # process-wide virtual setting of gpt_fast.tp
+    shard_vocab: Optional[bool] = None
 
     def __post_init__(self):
         if self.tp_world_size is None:
             self.tp_world_size = _tp.get_tp_world_size()
         if self.tp_rank is None:
             self.tp_rank = _tp.get_tp_rank() if self.tp_world_size == _tp.get_tp_world_size() else 0
+        if self.shard_vocab is None:
+            self.shard_vocab = _tp.get_shard_vocab() if self.tp_world_size == _tp.get_tp_world_size() else False
         if self.n_local_heads == -1:
             self.n_local_heads = self.n_head
         if self.intermediate_size is None:

@@ -6,8 +6,10 @@ setup_caches reads the model dtype from `output.scales` (gpt_ladder_TP.py:232-23
 provides that replacement for float8_e4m3fn and the quantiser; the forward is
     y = F.linear(x, weight.to(x.dtype)) * scales
 computed by lr_linear_fp8 (the fp8 bytes are streamed once: half the HBM traffic of bf16 decode).
-The one-kernel decode step reads bf16 weights, so a quantised model decodes through the per-op
-kernels."""
+A ladder model whose projections are all quantised (lm_head included) decodes at batch 1 and 2 through the
+one-kernel step on e4m3 weights (lr_ladder_decode_step_fp8; _hip.pack_fp8_linear lays a module's bytes and
+scales out the way it reads them); other batch sizes, other families and models with a bf16 lm_head go
+through the per-op fp8 kernels (lr_linear_fp8, lr_linear_fp8_multi, lr_attn_decode_beside_fp8)."""
 import torch
 import torch.nn as nn
 

@@ -9,14 +9,20 @@ import os
 from typing import Optional
 
 _TP_WORLD_SIZE = 1
+_SHARD_VOCAB = False
 _TP_RANK = 0
 
 
-def set_virtual_tp(world_size: int, rank: int = 0) -> None:
-    """Shard shapes as rank `rank` of `world_size` (layers are built at size // world_size)."""
-    global _TP_WORLD_SIZE, _TP_RANK
+def set_virtual_tp(world_size: int, rank: int = 0, shard_vocab: bool = False) -> None:
+    """Shard shapes as rank `rank` of `world_size` (layers are built at size // world_size).  shard_vocab: the
+    lm_head keeps vocab_size // world_size rows as well (the reference replicates the whole head on every rank)."""
+    global _TP_WORLD_SIZE, _TP_RANK, _SHARD_VOCAB
     assert world_size >= 1 and 0 <= rank < world_size
-    _TP_WORLD_SIZE, _TP_RANK = int(world_size), int(rank)
+    _TP_WORLD_SIZE, _TP_RANK, _SHARD_VOCAB = int(world_size), int(rank), bool(shard_vocab)
+
+
+def get_shard_vocab() -> bool:
+    return _SHARD_VOCAB
 
 
 def get_tp_world_size() -> int:

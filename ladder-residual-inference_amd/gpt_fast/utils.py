@@ -38,14 +38,24 @@ def is_flash_attention_enabled() -> bool:
 
 
 class KVCache(nn.Module):
-    """[max_batch, kv heads of this rank, max_seq, head_dim], zero-initialised, written in place by
-    lr_rope_kv_write."""
+    """[max_batch, kv heads of this rank, max_seq, head_dim], zero-initialised (utils.py:43-59).  The model's own
+    forward writes it in place from inside its projection kernels (lr_rope_kv_write and the RoPE + cache epilogues);
+    update() is the reference's method for callers that hold the module themselves."""
 
     def __init__(self, max_batch_size, max_seq_length, n_heads, head_dim, dtype=torch.bfloat16):
         super().__init__()
         shape = (max_batch_size, n_heads, max_seq_length, head_dim)
         self.register_buffer("k_cache", torch.zeros(shape, dtype=dtype))
         self.register_buffer("v_cache", torch.zeros(shape, dtype=dtype))
+
+    def update(self, input_pos: Tensor, k_val: Tensor, v_val: Tensor):
+        """k_cache[:, :, input_pos] = k_val ([B, H, S, D]), the same for v; returns (k_cache, v_cache) as the
+        reference does (utils.py:50-59).  One launch of lr_kv_update; positions stay on the device."""
+        assert input_pos.shape[0] == k_val.shape[2]
+        if k_val.stride(-1) != 1 or k_val.stride() != v_val.stride():
+            k_val, v_val = k_val.contiguous(), v_val.contiguous()
+        _hip.kv_update(k_val, v_val, input_pos.to(torch.int32), self.k_cache, self.v_cache)
+        return self.k_cache, self.v_cache
 
 
 class RMSNorm(nn.Module):

@@ -170,6 +170,28 @@ def test_virtual_tp_builds_one_rank_without_a_process_group(monkeypatch):
         maybe_init_dist()
 
 
+def test_shard_vocab_flag_reaches_the_model_shape():
+    """benchmark.py --virtual_tp N --shard_vocab: the lm_head of the unsharded registry names is built at
+    vocab_size / N rows (the reference's flag surface is benchmark.py:498-518; it replicates the head)."""
+    import benchmark as bm
+    from gpt_fast import tp
+    from gpt_fast.config import args_from_name
+
+    args = bm.build_parser().parse_args(["--model_name", "gpt_ladder:70B", "--prompt_length", "8", "--virtual_tp", "8",
+                                         "--shard_vocab"])
+    assert args.shard_vocab and args.virtual_tp == 8
+    tp.set_virtual_tp(args.virtual_tp, args.tp_rank, args.shard_vocab)
+    try:
+        c = args_from_name("ladder", "70B")
+        assert c.tp_world_size == 8 and c.shard_vocab and c.output_rows == c.vocab_size // 8
+        assert c.n_head_local == 8 and c.n_kv_local == 1 and c.ffn_local == 3584
+    finally:
+        tp.set_virtual_tp(1, 0)
+    c = args_from_name("ladder", "70B")
+    assert not c.shard_vocab and c.output_rows == c.vocab_size
+    assert not bm.build_parser().parse_args(["--model_name", "gpt_ladder:70B", "--prompt_length", "8"]).shard_vocab
+
+
 def test_bytes_per_step_accounting():
     import benchmark as bm
     from gpt_fast.config import args_from_name

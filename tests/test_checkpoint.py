@@ -118,6 +118,14 @@ def test_model_args_from_the_reference_hf_configs():
     assert a.ladder_layers == list(range(16, 32)) and a.rope_scaling["factor"] == 8.0 and a.rope_base == 500000.0
     assert not a.is_ladder_layer(15) and a.is_ladder_layer(16) and (a.n_head_local, a.ffn_local) == (4, 1792)
     assert ModelArgs(**model_args_from_hf_config(dict(hf, ladder_layers=32))).ladder_layers is None   # all layers
+    # no field at all (a plain Llama config.json) or null: NO ladder layer, every block dense
+    # (configuration_llama_ladder.py:38-39) -- not ModelArgs' own default of "all layers"
+    plain = {k: v for k, v in hf.items() if k != "ladder_layers"}
+    for cfg in (plain, dict(hf, ladder_layers=None)):
+        a0 = ModelArgs(**model_args_from_hf_config(cfg))
+        assert a0.ladder_layers == [] and not any(a0.is_ladder_layer(i) for i in range(a0.n_layer))
+    with pytest.raises(ValueError):
+        model_args_from_hf_config(dict(hf, ladder_layers="16"))
     with pytest.raises(ValueError):
         model_args_from_hf_config(dict(hf, rope_scaling={"rope_type": "yarn", "factor": 2.0}))
 
@@ -171,18 +179,18 @@ def test_hip_model_serves_a_loaded_hf_checkpoint(tmp_path, tp, rank, ladder_laye
     from gpt_fast.config import ModelArgs
     from safetensors.torch import save_file
 
-    shape = dict(n_layer=4, n_head=4, n_kv=2, dim=256, ffn=384, vocab=320)
+    shape = dict(n_layer=4, n_head=4, n_kv=2, dim=256, ffn=512, vocab=320)
     hf = random_hf_state_dict(**shape, seed=11, dtype=torch.bfloat16)
     path = str(tmp_path / "model.safetensors")
     save_file(hf, path)
-    kw = dict(block_size=64, vocab_size=320, n_layer=4, n_head=4, n_local_heads=2, dim=256, intermediate_size=384,
+    kw = dict(block_size=64, vocab_size=320, n_layer=4, n_head=4, n_local_heads=2, dim=256, intermediate_size=512,
               rope_base=10000, tp_world_size=tp, tp_rank=rank, shard_vocab=tp > 1, ladder_layers=ladder_layers)
     with torch.device("meta"):
         model = bm.GPTLadder(ModelArgs(**kw))
     model = model.to(dtype=torch.bfloat16).to_empty(device="cuda").eval()
     load_checkpoint(model, path)
     cfg = model.config
-    ocfg = O.OracleConfig(block_size=64, vocab_size=320, n_layer=4, n_head=4, n_local_heads=2, dim=256, intermediate_size=384,
+    ocfg = O.OracleConfig(block_size=64, vocab_size=320, n_layer=4, n_head=4, n_local_heads=2, dim=256, intermediate_size=512,
                           rope_base=10000, tp_world_size=tp, vocab_shard=cfg.output_rows if tp > 1 else None,
                           ladder_layers=cfg.ladder_layers)
     P = dict(model.state_dict())

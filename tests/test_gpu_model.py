@@ -354,6 +354,31 @@ def test_fused_step_every_instance(B, hd, G, fp8):
     assert stats["fused_step_used"]
 
 
+def test_fused_step_is_refused_unless_every_workgroup_can_be_resident():
+    """The step launches one workgroup per compute unit and they wait for each other: the library reports how many
+    workgroups of the instance the device can hold for a descriptor (occupancy x compute units), refuses the
+    launch below one per compute unit, and reports 0 for shapes the step does not serve."""
+    import ctypes
+
+    from gpt_fast import _hip
+
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    lib = _hip.load()
+    big = build("ladder", **dict(TINY, block_size=2200, n_head=8, n_local_heads=1, dim=1024, intermediate_size=3584,
+                                 n_layer=1))     # the rank shard's head layout: the 70B instance, LDS sized by ffn
+    big.setup_caches(1, 2112)
+    fs = _hip.FusedLadderStep(big, 1)
+    assert fs.supported and fs.resident >= cus
+    assert lib.lr_ladder_step_resident_workgroups(ctypes.byref(fs.desc), 1) == fs.resident      # remembered per device
+    assert lib.lr_ladder_step_resident_workgroups(ctypes.byref(fs.desc), 3) == 0                 # no instance for batch 3
+    # fewer q/k/v rows than compute units: some workgroup would own no row of the projection that orders the
+    # exchange arrays -- left to the per-op kernels
+    thin = build("ladder", **dict(TINY, n_head=1, n_local_heads=1, dim=64, intermediate_size=512, n_layer=1))
+    thin.setup_caches(1, 64)
+    assert (1 + 2) * 64 < cus
+    assert not _hip.FusedLadderStep(thin, 1).supported
+
+
 def test_fused_step_head_dim_64_longest_key_range_per_workgroup():
     """head_dim 64 with a cache of 8160 slots: 16 attention workgroups of 510 keys each, the most a
     workgroup's score tiles cover (2 x 8 waves x 32 keys = 512).  Beyond that the step must refuse."""

@@ -369,6 +369,42 @@ def test_rope_kv_write_exact(hip, hd, Hq, Hkv, gathered):
     assert torch.equal(work[..., Hq * hd:], torch.cat([k, v], -1))   # k and v columns are left as they were
 
 
+@pytest.mark.parametrize("hd,H", [(128, 1), (64, 8), (128, 8)])
+@pytest.mark.parametrize("layout", ["bhsd", "bshd"])
+def test_kv_cache_update_module_method(hd, H, layout):
+    """KVCache.update (utils.py:50-59) through lr_kv_update: dense [B, H, S, D] values and the transposed view of a
+    [B, S, H, D] tensor (what a caller holds right after splitting a projection), scattered positions, a batch
+    smaller than the cache; bit-exact against the oracle's indexed assignment, rows not addressed stay zero."""
+    from gpt_fast.utils import KVCache
+
+    B, S, Smax = 2, 7, 40
+    pos = torch.tensor([0, 5, 6, 7, 21, 38, 39], device=DEV)          # int64, as torch.arange gives
+    if layout == "bhsd":
+        k, v = rnd(B, H, S, hd, seed=70), rnd(B, H, S, hd, seed=71)
+    else:
+        k, v = rnd(B, S, H, hd, seed=70).transpose(1, 2), rnd(B, S, H, hd, seed=71).transpose(1, 2)
+    cache = KVCache(B + 1, Smax, H, hd).to(DEV)
+    kc_ref, vc_ref = cache.k_cache.clone(), cache.v_cache.clone()
+    O.kv_update(kc_ref, vc_ref, pos, k, v)
+    k_out, v_out = cache.update(pos, k, v)
+    assert k_out is cache.k_cache and v_out is cache.v_cache
+    assert torch.equal(k_out, kc_ref) and torch.equal(v_out, vc_ref)
+    assert float(k_out[B].abs().max()) == 0.0 and float(k_out[:, :, 1].abs().max()) == 0.0
+
+
+def test_kv_cache_update_reports_a_position_outside_the_cache(hip):
+    from gpt_fast.utils import KVCache
+
+    cache = KVCache(1, 16, 2, 64).to(DEV)
+    k = rnd(1, 2, 2, 64, seed=72)
+    hip.device_error_word(DEV).zero_()
+    cache.update(torch.tensor([3, 16], device=DEV), k, k)
+    torch.cuda.synchronize()
+    assert int(hip.device_error_word(DEV).item()) == 2            # LR_DEV_POS_RANGE; slot 3 was still written
+    assert torch.equal(cache.k_cache[0, :, 3], k[0, :, 0])
+    hip.device_error_word(DEV).zero_()
+
+
 @pytest.mark.parametrize("rows,dim", [(1, 8192), (8, 8192), (64, 4096), (3, 2048), (16, 16384), (5, 264)])
 @pytest.mark.parametrize("first_block", [False, True])
 def test_ladder_norms_equals_two_add_rmsnorm_calls(hip, rows, dim, first_block):
