@@ -595,6 +595,20 @@ def test_ladder_70b_tp8_shard_shape_with_fp8_weights(B):
     check(stats)
 
 
+@pytest.mark.parametrize("B", [1, 8])
+def test_ladder_70b_tp8_shard_config3_full_with_fp8_weights(B):
+    """Config 3 at its full size (80 layers, prompt 2048) in the weight-only fp8 form: batch 1 through the
+    one-kernel step on e4m3 weights, batch 8 through the fp8 bands."""
+    from gpt_fast.quantize import quantize_model_fp8
+
+    progress(f"cfg3 fp8 B={B}: building")
+    model = quantize_model_fp8(build("ladder", **shape_kw("ladder-70b-tp8")))
+    stats = run_parity(model, "ladder", B=B, T=2048, new=32)
+    report(f"fp8 weights, cfg3 ladder-70b-tp8, 80 layers, B={B}", stats)
+    check(stats)
+    assert stats["fused_step_used"] == (B == 1)
+
+
 # ---------------------------------------------------------------------------------------------------
 # token identity with teeth: weights under which the greedy token changes from step to step
 # ---------------------------------------------------------------------------------------------------
@@ -637,10 +651,12 @@ CONDITIONED_PROMPT_SEED = 21   # a prompt for which the oracle's token stream mo
 
 
 @torch.no_grad()
-@pytest.mark.parametrize("B", [1, 8])
-def test_ladder_70b_tp8_shard_tokens_on_conditioned_weights(B):
-    """The 70B rank shard at its full size with well-conditioned weights, where the oracle's greedy
-    tokens change from step to step, so that "tokens identical" can fail.
+@pytest.mark.parametrize("name,B,T", [("ladder-70b-tp8", 1, 2048), ("ladder-70b-tp8", 8, 2048), ("ladder-8b", 16, 1024)])
+def test_tokens_on_conditioned_weights(name, B, T):
+    """The 70B rank shard (batch 1: the one-kernel step; batch 8: the bands with the attention beside up/gate) and the
+    8B model (batch 16: eight kv heads per rank, the attention items of all of them beside the up/gate bands) at
+    their full size with well-conditioned weights, where the oracle's greedy tokens change from step to step, so
+    that "tokens identical" can fail.
 
     With activations of order one in all 80 layers bf16 arithmetic is itself noisy: the eager bf16
     oracle differs from the SAME oracle run in fp32 by ~1e-1 of the largest logit, and two bf16
@@ -655,8 +671,8 @@ def test_ladder_70b_tp8_shard_tokens_on_conditioned_weights(B):
         the hipGraph replay equals the eager generation token for token."""
     import benchmark as bm
 
-    T, new = 2048, 48
-    model = build("ladder", **shape_kw("ladder-70b-tp8"))
+    new = 48
+    model = build("ladder", **shape_kw(name))
     init_conditioned(model, seed=0)
     cfg, ocfg = model.config, oracle_cfg(model.config)
     P = dict(model.state_dict())
@@ -664,7 +680,7 @@ def test_ladder_70b_tp8_shard_tokens_on_conditioned_weights(B):
     g.manual_seed(CONDITIONED_PROMPT_SEED)
     prompt = torch.randint(0, cfg.vocab_size, (T,), device=DEV, generator=g)
     model.setup_caches(B, T + new)
-    progress(f"conditioned weights B={B}: oracle generation (bf16, then fp32 on the same tokens)")
+    progress(f"conditioned weights {name} B={B}: oracle generation (bf16, then fp32 on the same tokens)")
     ref_tok, ref_logits = O.generate(ocfg, P, prompt, new, B, "ladder")
     P32 = {k: v.float() for k, v in P.items()}
     _, exact_logits = O.generate(ocfg, P32, prompt, new, 1, "ladder", forced=ref_tok[:1])
@@ -692,7 +708,7 @@ def test_ladder_70b_tp8_shard_tokens_on_conditioned_weights(B):
         pos += 1
     forced = torch.cat(forced, dim=1)
     same = forced == ref_tok
-    line = (f"conditioned weights B={B}: tokens identical at {float(same.float().mean()):.4f} of all steps, at "
+    line = (f"conditioned weights {name} B={B}: tokens identical at {float(same.float().mean()):.4f} of all steps, at "
             f"{float(same[robust].float().mean()):.4f} of the robust ones; distance to the fp32 logits: HIP {max(errs):.3e}, "
             f"eager bf16 oracle {oracle_err:.3e}")
     progress(line)
@@ -774,6 +790,16 @@ def test_variants_on_70b_shard_shape(family, B):
                   force_disable_last_all_reduce=True)
     stats = run_parity(build(family, **kw), family, B=B, T=300, new=10)
     report(f"{family} on the 70B shard shape, B={B}", stats)
+    check(stats)
+
+
+@pytest.mark.parametrize("family,B", [("dense", 1), ("dense", 8), ("parallel", 1), ("parallel", 8)])
+def test_variants_on_70b_shard_shape_at_full_depth(family, B):
+    """Dense and parallel blocks (gpt_dense_TP.py:274-284, gpt_parallel_TP.py:214-226) on the 70B rank shard's
+    matrices at all 80 layers, prompt 2048: what 80 layers of bf16 rounding do to the logits stays within the bar."""
+    progress(f"{family} at 80 layers B={B}: building")
+    stats = run_parity(build(family, **shape_kw("ladder-70b-tp8")), family, B=B, T=2048, new=24)
+    report(f"{family} on the 70B shard shape, 80 layers, B={B}", stats)
     check(stats)
 
 
