@@ -67,12 +67,15 @@ def build(force=False, verbose=True):
 
 
 def build_step_profile(force=False, verbose=True):
-    """A second library, gpt_fast/libladder_hip_prof.so, whose decode-step kernel records wall-clock stamps per
-    workgroup and phase (-DLR_STEP_PROFILE; read by step_phases.py).  The product library carries none of it."""
+    """A second library, gpt_fast/libladder_hip_prof.so, whose decode-step kernels (bf16 and e4m3 weights) record
+    wall-clock stamps per workgroup and phase (-DLR_STEP_PROFILE; read by step_phases.py).  The product library
+    carries none of it."""
     build(force=force, verbose=False)
-    obj, changed = _compile(os.path.join(CSRC, "ladder_step.hip"), force, ("-DLR_STEP_PROFILE",), "_prof")
+    step_sources = ("ladder_step.hip", "ladder_step_fp8.hip")
+    res = [_compile(os.path.join(CSRC, f), force, ("-DLR_STEP_PROFILE",), "_prof") for f in step_sources]
+    changed = any(c for _, c in res)
     objs = [os.path.join(OBJ, f.replace(".hip", ".o")) for f in sorted(os.listdir(CSRC))
-            if f.endswith(".hip") and f != "ladder_step.hip"] + [obj]
+            if f.endswith(".hip") and f not in step_sources] + [o for o, _ in res]
     if force or changed or _stale(PROF_LIB, objs):
         r = subprocess.run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PROF_LIB] + objs,
                            capture_output=True, text=True)

@@ -736,15 +736,17 @@ __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, con
   for (int j0 = 0; j0 < job.nj; j0 += NJMAX) {
     const int njb = job.nj - j0 < NJMAX ? job.nj - j0 : NJMAX;
 #if LR_STEP_W8
-    // the scales of the outputs this lane will finish are requested now: their round trip is over when the
-    // round's units have been multiplied
-    float sc0 = 1.0f, sc1 = 1.0f;
+    // The scales of the outputs this lane will finish are requested now: their round trip is over when the
+    // round's units have been multiplied.  They stay raw bits until then: converted here, the conversion (and with
+    // it a wait for the load, the youngest in flight, i.e. for everything) would sit at the top of every job.
+    u32 sraw0 = 0x3f80, sraw1 = 0x3f80;  // 1.0
     if (tid < (njb >> job.rsh) * M) {
       const int it_s = job.first + (j0 >> job.rsh) + tid / M;
-      sc0 = bf_to_f(job.S[it_s]);
-      if (EPI == EPI_SWIGLU) sc1 = bf_to_f(job.S[it_s + job.pair_off]);
+      sraw0 = gld2(job.S + it_s);
+      if (EPI == EPI_SWIGLU) sraw1 = gld2(job.S + it_s + job.pair_off);
     }
 #endif
+    if (stamp && tid == 0 && (sb == 16 || sb == 20)) stamp[sb == 16 ? 30 : 31] = wall_clock64();
     if (job.active && job.rg < njb) {
       const int up = c.up;
       for (int u = 0; u < up; u += 2) {
@@ -780,8 +782,9 @@ __device__ __forceinline__ void run_job(const StepParams& p, const Coh& coh, con
         if (EPI == EPI_SWIGLU) s1 = round_bf(t1);
       }
 #if LR_STEP_W8
-      s0 = round_bf(s0 * sc0);
-      s1 = round_bf(s1 * sc1);
+      asm volatile("" : "+v"(sraw0), "+v"(sraw1));  // (the conversion stays down here)
+      s0 = round_bf(s0 * __uint_as_float(sraw0 << 16));
+      s1 = round_bf(s1 * __uint_as_float(sraw1 << 16));
 #endif
       const int it = job.first + (j0 >> job.rsh) + jl;
       if (m < p.B) {
@@ -1700,10 +1703,16 @@ int g_prof_t0 = 0;
 }  // namespace
 
 #ifdef LR_STEP_PROFILE
-// Debug builds only (not declared in the public header): following steps record, per workgroup,
+// Profile builds only (not declared in the public header): following steps record, per workgroup,
 // wall-clock stamps (100 MHz) for PROF_SLOTS consecutive slots starting at `first_slot` into
-// `device_buffer` (NULL switches it off).  Returns the bytes the buffer must hold.
-extern "C" size_t lr_ladder_step_profile(void* device_buffer, int first_slot) {
+// `device_buffer` (NULL switches it off).  Returns the bytes the buffer must hold.  The e4m3 instance has a
+// hook of its own (lr_ladder_step_profile_fp8).
+#if LR_STEP_W8
+#define LR_PROFILE_ENTRY lr_ladder_step_profile_fp8
+#else
+#define LR_PROFILE_ENTRY lr_ladder_step_profile
+#endif
+extern "C" size_t LR_PROFILE_ENTRY(void* device_buffer, int first_slot) {
   g_prof = reinterpret_cast<unsigned long long*>(device_buffer);
   g_prof_t0 = first_slot;
   return (size_t)lr_num_cus() * PROF_SLOTS * PROF_POINTS * sizeof(unsigned long long);

@@ -46,6 +46,9 @@ __device__ __forceinline__ uint4 gld16(const void* p) {
   const u32x4_t v = *(const __attribute__((address_space(1))) u32x4_t*)((unsigned long long)p);
   return make_uint4(v.x, v.y, v.z, v.w);
 }
+__device__ __forceinline__ u16 gld2(const void* p) {
+  return *(const __attribute__((address_space(1))) u16*)((unsigned long long)p);
+}
 __device__ __forceinline__ void gst4(void* p, u32 v) {
   *(__attribute__((address_space(1))) u32*)((unsigned long long)p) = v;
 }

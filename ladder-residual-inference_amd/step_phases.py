@@ -40,6 +40,7 @@ def main():
     ap.add_argument("--slot", type=int, default=40, help="first of the four layer slots that are stamped")
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--batch", type=int, default=1, choices=(1, 2))
+    ap.add_argument("--fp8", action="store_true", help="weight-only e4m3 projections: the one-kernel step on e4m3 weights")
     ap.add_argument("--lib", default=os.path.join(HERE, "gpt_fast", "libladder_hip_prof.so"),
                     help="the profile build of the library")
     args = ap.parse_args()
@@ -51,13 +52,18 @@ def main():
     import benchmark as bm
 
     model = bm._load_model(args.model, "cuda", torch.bfloat16, seed=0, verbose=False)
+    if args.fp8:
+        from gpt_fast.quantize import quantize_model_fp8
+
+        quantize_model_fp8(model)
     T = args.prompt
     B = args.batch
     model.setup_caches(B, T + 64)
     model.last_logits_only = True
     lib = _hip.load()
-    lib.lr_ladder_step_profile.restype = ctypes.c_size_t
-    lib.lr_ladder_step_profile.argtypes = [ctypes.c_void_p, ctypes.c_int]
+    set_profile = lib.lr_ladder_step_profile_fp8 if args.fp8 else lib.lr_ladder_step_profile
+    set_profile.restype = ctypes.c_size_t
+    set_profile.argtypes = [ctypes.c_void_p, ctypes.c_int]
     with torch.no_grad():
         prompt = torch.randint(0, model.config.vocab_size, (T,), device="cuda")
         first = bm.prefill(model, prompt.view(1, -1).repeat(B, 1), torch.arange(T, device="cuda", dtype=torch.int32),
@@ -65,9 +71,9 @@ def main():
         pos = torch.tensor([T], dtype=torch.int32, device="cuda")
         for _ in range(3):
             model(first.view(B, 1), pos)
-        nbytes = lib.lr_ladder_step_profile(None, 0)
+        nbytes = set_profile(None, 0)
         buf = torch.zeros(nbytes // 8, dtype=torch.int64, device="cuda")
-        lib.lr_ladder_step_profile(buf.data_ptr(), args.slot)
+        set_profile(buf.data_ptr(), args.slot)
         # two single stamped steps first: are the same workgroups slow in the same slot of different steps?
         snaps = []
         for _ in range(2):
@@ -80,9 +86,9 @@ def main():
             model(first.view(B, 1), pos)
         e1.record()
         torch.cuda.synchronize()
-        lib.lr_ladder_step_profile(None, 0)
+        set_profile(None, 0)
     model.check_device_errors()
-    print(f"{args.model}, batch {B}, position {T}: {e0.elapsed_time(e1) / args.steps:.3f} ms per step (profile build, eager launches)")
+    print(f"{args.model}{' (e4m3 weights)' if args.fp8 else ''}, batch {B}, position {T}: {e0.elapsed_time(e1) / args.steps:.3f} ms per step (profile build, eager launches)")
     NP = 32   # stamps per workgroup and slot (PROF_POINTS of the kernel)
     a = buf.cpu().numpy().reshape(-1, 4, NP).astype(np.float64) * 0.01   # [workgroup][slot][stamp] in microseconds
     nwg = a.shape[0]
@@ -103,6 +109,9 @@ def main():
     for nm, (k0, k1, k2) in JOB_PARTS.items():
         d0, d1 = (a[na:, :, k1] - a[na:, :, k0]).mean(axis=1), (a[na:, :, k2] - a[na:, :, k1]).mean(axis=1)
         print(f"    {nm:42s} mean {d0.mean():6.2f} | {d1.mean():5.2f}   max {d0.max():6.2f} | {d1.max():5.2f}")
+    for nm, k0, k1 in (("wqkv: entry -> first unit wanted", 1, 30), ("wo: entry -> first unit wanted", 5, 31)):
+        d = (a[na:, :, k1] - a[na:, :, k0]).mean(axis=1)
+        print(f"    {nm:42s} mean {d.mean():6.2f}   max {d.max():6.2f}")
     cnt = buf.cpu().numpy().reshape(-1, 4, NP)[:, :, 24:30].sum(axis=(0, 1)) / (4.0 * args.steps)
     print("  exchanged words not there at the first look, per slot, summed over the workgroups: "
           + ", ".join(f"{n} {c:.1f}" for n, c in zip(STALE_NAMES, cnt)))
