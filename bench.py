@@ -16,7 +16,8 @@ Prints ONE JSON line.  `value` = decoded tokens per second (whole job = the one 
                launch duration, measured here with HIP events around back-to-back launches on the
                launch stream.  `traffic` = HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE
                counter runs (a constant recorded from those runs, or null).  Other models / batches
-               fall back to the per-op path, whose dominant kernel is the w1 GEMV.
+               run the per-op path, whose dominant kernel is the up/gate projection (timed alone here:
+               the GEMV up to batch 4, the matrix-core band kernel above).
                `measured_read_ceiling` = GB/s of a plain streaming read of 8 GiB by every CU
                (lr_stream_read) on this machine in the same run; `frac` is against the nominal
                8 TB/s, `frac_of_measured_ceiling` against that.
@@ -30,7 +31,8 @@ Prints ONE JSON line.  `value` = decoded tokens per second (whole job = the one 
 Measured in the same run and reported as extra keys (not the headline; --no-extras skips them):
 `batched`     : the same rank shard at batch 8 and 64, the 8B model at batch 1 (one-kernel step) and 16 (prompt
                1024) and the 405B rank shard at batch 16 (context 4096) -- per-op kernels unless noted,
-               hipGraph replay: ms per step, tok/s, algorithmic GB/s and its fraction of 8 TB/s.
+               hipGraph replay: ms per step, tok/s, algorithmic GB/s and its fraction of 8 TB/s; `traffic` = HBM
+               bytes per step from counter runs where one was made.
 `fp8`         : the same shard with weight-only e4m3 projections at batch 1 (the one-kernel step on e4m3 weights)
                and batch 8 (per-op kernels): ms per step and the fraction of 8 TB/s on ITS algorithmic bytes
                (one byte per weight + scales).
@@ -50,7 +52,17 @@ HBM_PEAK_GBPS = 8000.0
 MFMA_PEAK_TFLOPS = 2500.0   # dense bf16
 # HBM bytes one launch of the dominant kernel moves, per workload (model, batch, prompt), from the rocprofv3
 # FETCH_SIZE / WRITE_SIZE counter runs summarised under profiles/; workloads without a counter run report null.
-TRAFFIC_BYTES_PER_LAUNCH = {("gpt_ladder:ladder-70b-tp8", 1, 2048): 17.65e9}   # 1.011 x algorithmic
+TRAFFIC_BYTES_PER_LAUNCH = {
+    ("gpt_ladder:ladder-70b-tp8", 1, 2048): 17.585e9,    # k_ladder_step, 1.007 x algorithmic
+    # the up/gate projection alone (the kernel the batched workloads' roofline object is measured on):
+    ("gpt_ladder:ladder-70b-tp8", 8, 2048): 118.75e6,    # k_stream_gemm<16,2>, 256 bands: 1.009 x algorithmic
+    ("gpt_ladder:ladder-70b-tp8", 64, 2048): 126.46e6,   # k_stream_gemm<64,2>, the decode step's 224 bands: 1.06 x
+}
+# HBM bytes of a whole decode step through the per-op kernels (all its launches), from the same kind of counter runs
+STEP_TRAFFIC_BYTES = {
+    ("gpt_ladder:ladder-70b-tp8", 8, 2048): 22.41e9,     # 1.24 x algorithmic
+    ("gpt_ladder:ladder-70b-tp8", 64, 2048): 30.46e9,    # 1.34 x algorithmic
+}
 
 
 def cpu_baseline(new_tokens=32, repeats=2):
@@ -120,7 +132,8 @@ def extra_batched(bm, model, prompt, T, batches=(4, 8, 64), K=32, W=5):
         gbps = nbytes / (ms * 1e-3) / 1e9
         out.append({"model": "gpt_ladder:ladder-70b-tp8", "batch": B, "prompt_len": T, "ms_per_step": round(ms, 4),
                     "tok_per_s": round(B * 1e3 / ms, 1), "bytes_per_step": int(nbytes), "achieved_GBps": round(gbps, 1),
-                    "frac": round(gbps / HBM_PEAK_GBPS, 4), "steps": K})
+                    "frac": round(gbps / HBM_PEAK_GBPS, 4), "steps": K,
+                    "traffic": STEP_TRAFFIC_BYTES.get(("gpt_ladder:ladder-70b-tp8", B, T))})
         del dg
     return out
 
@@ -378,7 +391,7 @@ def main():
         "roofline": {"bound": "hbm", "kernel": k_name,
                      "achieved": round(k_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(k_gbps / HBM_PEAK_GBPS, 4),
-                     "traffic": TRAFFIC_BYTES_PER_LAUNCH.get((args.model, B, T)) if fused and not args.fp8 else None,
+                     "traffic": TRAFFIC_BYTES_PER_LAUNCH.get((args.model, B, T)) if (fused or B > 4) and not args.fp8 else None,
                      "bytes_per_launch": int(k_bytes), "avg_launch_us": round(k_us, 3),
                      "measured_read_ceiling": round(ceiling_gbps, 1),
                      "frac_of_measured_ceiling": round(k_gbps / ceiling_gbps, 4)},
