@@ -167,9 +167,16 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
 
   const int nck = (K + KCW - 1) / KCW;
   const int nch = wave < nck ? (nck - wave + NWV - 1) / NWV : 0;  // chunks of this wave
+  // (the fences keep the requests in this order: the wait for chunk 0 counts the requests made after it, and the
+  // scheduler, left alone, asks for chunk 0 last -- the loop then waited for all but the last 8 requests at the top
+  // of every round of NS chunks)
   issue_x(0, xr[0]);
 #pragma unroll
-  for (int s = 0; s < NS; ++s) issue_w(s, wr[s]);
+  for (int s = 0; s < NS; ++s) {
+    asm volatile("" ::: "memory");
+    issue_w(s, wr[s]);
+  }
+  asm volatile("" ::: "memory");
   for (int c0 = 0; c0 < nch; c0 += NS) {
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
