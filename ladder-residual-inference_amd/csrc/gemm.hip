@@ -280,60 +280,66 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
 
   // The products were formed as W-tile x X-tile^T, so accumulator element v of a 32 x 32 tile is
   // output column n = (v / 4) * 8 + (lane / 32) * 4 + v % 4 of output row m = lane % 32: a lane holds
-  // four consecutive n of one row per group of four registers -> one 8-byte store.
-  const bool vec_ok = (ldy & 3) == 0;
-  if (pair_off) {
+  // four consecutive n of one row per group of four registers.  Stored from there, an instruction would
+  // touch 16 bytes in each of 32 rows (32 partial cache lines, every line eight times per tile): the
+  // tile's outputs take one trip through LDS instead (the operand tiles are dead; every wave has a piece
+  // of its own) and leave as whole rows, an instruction covering 256 contiguous bytes of each of 4 rows
+  // (128 bytes of 8 rows in pair mode).
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // nobody still reads the operand tiles
+  u16* const eb = gsm + wave * (128 * (128 + 8));
+  auto emit = [&](auto PAIR) {
+    int lane = threadIdx.x & 63;  // (laundered: the addresses below are not formed before the k loop and kept through it)
+    asm volatile("" : "+v"(lane));
+    constexpr bool P = decltype(PAIR)::value;
+    constexpr int WN = P ? 64 : 128;   // output columns of a wave
+    constexpr int EP = WN + 8;         // row pitch of the wave's piece, in elements
+    constexpr int LPR = WN / 8;        // lanes per row in the read-back
+    constexpr int RPI = 64 / LPR;      // rows per instruction
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
-      const int m = m0 + wm * 128 + a * 32 + (lane & 31);
+      const int ml = a * 32 + (lane & 31);
 #pragma unroll
-      for (int b = 0; b < 2; ++b) {
+      for (int b = 0; b < (P ? 2 : 4); ++b)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          const int n = n0 + wn * 64 + b * 32 + g * 8 + (lane >> 5) * 4;
-          if (m < M) {
+          const int nl = b * 32 + g * 8 + (lane >> 5) * 4;
+          uint2 pk;
+          if constexpr (P) {
             float o[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) o[e] = swiglu_bf(round_bf(acc[a][b][4 * g + e]), round_bf(acc[a][b + 2][4 * g + e]));
-            if (vec_ok && n + 3 < N) {
-              uint2 pk;
-              pk.x = pack_bf2(o[0], o[1]);
-              pk.y = pack_bf2(o[2], o[3]);
-              *reinterpret_cast<uint2*>(y + (int64_t)m * ldy + n) = pk;
-            } else {
-#pragma unroll
-              for (int e = 0; e < 4; ++e)
-                if (n + e < N) y[(int64_t)m * ldy + n + e] = f_to_bf(o[e]);
-            }
-          }
-        }
-      }
-    }
-    return;
-  }
-#pragma unroll
-  for (int a = 0; a < 4; ++a) {
-    const int m = m0 + wm * 128 + a * 32 + (lane & 31);
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int n = n0 + wn * 128 + b * 32 + g * 8 + (lane >> 5) * 4;
-        if (m < M) {
-          if (vec_ok && n + 3 < N) {
-            uint2 pk;
+            pk.x = pack_bf2(o[0], o[1]);
+            pk.y = pack_bf2(o[2], o[3]);
+          } else {
             pk.x = pack_bf2(acc[a][b][4 * g], acc[a][b][4 * g + 1]);
             pk.y = pack_bf2(acc[a][b][4 * g + 2], acc[a][b][4 * g + 3]);
-            *reinterpret_cast<uint2*>(y + (int64_t)m * ldy + n) = pk;
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (n + e < N) y[(int64_t)m * ldy + n + e] = f_to_bf(acc[a][b][4 * g + e]);
           }
+          *reinterpret_cast<uint2*>(&eb[ml * EP + nl]) = pk;
+        }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // a wave reads back only what it wrote itself
+    const bool vec_ok = (ldy & 7) == 0;
+    const int cl = (lane % LPR) * 8;
+    const int ncol0 = n0 + wn * WN + cl;
+#pragma unroll 4
+    for (int r0 = 0; r0 < 128; r0 += RPI) {
+      const int ml = r0 + lane / LPR;
+      const int m = m0 + wm * 128 + ml;
+      const uint4 v = *reinterpret_cast<const uint4*>(&eb[ml * EP + cl]);
+      if (m < M) {
+        if (vec_ok && ncol0 + 7 < N) {
+          *reinterpret_cast<uint4*>(y + (int64_t)m * ldy + ncol0) = v;
+        } else {
+          const u32 q[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (ncol0 + e < N) y[(int64_t)m * ldy + ncol0 + e] = (u16)(q[e >> 1] >> ((e & 1) * 16));
         }
       }
     }
-  }
+  };
+  if (pair_off) emit(std::true_type{});
+  else emit(std::false_type{});
 }
 
 // pair_off != 0: N counts [up; gate] row pairs (see the kernel)
