@@ -221,7 +221,9 @@ def test_step_descriptor_is_validated_on_the_host(lib):
     import ctypes
 
     E_NULL, E_SHAPE, E_UNSUPPORTED = -1, -3, -4
-    init = lambda d, b=1: lib.lr_ladder_step_init(ctypes.byref(d), b, 256, 1 << 20, None)
+    # (the workspace pointer is misaligned on purpose: where a GPU is present a descriptor that passes validation is
+    # then refused with LR_E_ALIGN instead of being initialised at a made-up address)
+    init = lambda d, b=1: lib.lr_ladder_step_init(ctypes.byref(d), b, 8, 1 << 20, None)
     # a cache longer than the RoPE table: positions beyond block_size would read past the end of freqs_cis
     assert init(_desc(smax=72, block_size=64)) == E_SHAPE
     assert lib.lr_ladder_step_workspace_bytes(ctypes.byref(_desc(smax=72, block_size=64)), 1) == 0
