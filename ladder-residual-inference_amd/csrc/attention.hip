@@ -30,7 +30,7 @@ __global__ __launch_bounds__(256) void k_attn_decode_partial(const u16* __restri
                                                              float* __restrict__ o_part, float* __restrict__ ml_part,
                                                              int Hkv, int Smax, int nsplit, int chunk_max) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  attn_partial_item<HD, G>(q, ldq, kc, vc, pos_ptr, o_part, ml_part, Hkv, Smax, nsplit, chunk_max, blockIdx.x,
+  attn_partial_item<HD, G, true>(q, ldq, kc, vc, pos_ptr, o_part, ml_part, Hkv, Smax, nsplit, chunk_max, blockIdx.x,
                            blockIdx.y, blockIdx.z, smem);
 }
 

@@ -36,13 +36,14 @@ struct AttnItems {
 
 constexpr int PAIR_MT = 16, PAIR_UNITS = 2;
 
-template <int HD, int G, bool W8, bool XL>
+// EAGER: how an attention item requests its rows (see attn_partial_item): all at once for long chunks
+template <int HD, int G, bool W8, bool XL, bool EAGER>
 __global__ __launch_bounds__(256) void k_attn_beside_band(const AttnItems a, const Proj p, const int M) {
   extern __shared__ __attribute__((aligned(16))) unsigned char pair_smem[];
   const int wg = blockIdx.x;
   if (wg < a.n_items) {
     const int split = wg % a.nsplit, rest = wg / a.nsplit;
-    attn_partial_item<HD, G>(a.q, a.ldq, a.kc, a.vc, a.pos, a.o_part, a.ml_part, a.Hkv, a.Smax, a.nsplit,
+    attn_partial_item<HD, G, EAGER>(a.q, a.ldq, a.kc, a.vc, a.pos, a.o_part, a.ml_part, a.Hkv, a.Smax, a.nsplit,
                              a.chunk_max, split, rest % a.Hkv, rest / a.Hkv, reinterpret_cast<float*>(pair_smem),
                              a.kv_share);
   } else {
@@ -50,15 +51,15 @@ __global__ __launch_bounds__(256) void k_attn_beside_band(const AttnItems a, con
   }
 }
 
-template <int HD, int G, bool W8, bool XL>
+template <int HD, int G, bool W8, bool XL, bool EAGER>
 static int launch_pair_as(const AttnItems& a, const Proj& p, int M, u16* y, int64_t ldy, int B, hipStream_t s) {
   const int Hq = a.Hkv * G;
   const size_t lds_att = (size_t)attn_item_lds_floats<HD, G>(a.chunk_max) * sizeof(float);
   const size_t lds_band = stream_band_lds_bytes<PAIR_MT, PAIR_UNITS, W8, XL>();
   const size_t lds = lds_att > lds_band ? lds_att : lds_band;
   static std::atomic<unsigned long long> lds_raised{0};
-  if (!lr_raise_lds_limit(reinterpret_cast<const void*>(&k_attn_beside_band<HD, G, W8, XL>), lds, lds_raised)) return LR_E_LAUNCH;
-  k_attn_beside_band<HD, G, W8, XL><<<dim3((unsigned)(a.n_items + p.nwg)), dim3(256), lds, s>>>(a, p, M);
+  if (!lr_raise_lds_limit(reinterpret_cast<const void*>(&k_attn_beside_band<HD, G, W8, XL, EAGER>), lds, lds_raised)) return LR_E_LAUNCH;
+  k_attn_beside_band<HD, G, W8, XL, EAGER><<<dim3((unsigned)(a.n_items + p.nwg)), dim3(256), lds, s>>>(a, p, M);
   k_attn_decode_combine<HD><<<dim3(Hq, B), dim3(HD), 0, s>>>(a.o_part, a.ml_part, y, ldy, Hq, a.nsplit);
   return lr_launch_status();
 }
@@ -66,8 +67,12 @@ static int launch_pair_as(const AttnItems& a, const Proj& p, int M, u16* y, int6
 // (the band's inputs in whole lines or in fragment layout: the choice lr_linear_multi makes for the same rows)
 template <int HD, int G, bool W8>
 static int launch_pair(const AttnItems& a, const Proj& p, int M, u16* y, int64_t ldy, int B, hipStream_t s) {
-  if (!W8 && M >= XLDS_M16_FROM) return launch_pair_as<HD, G, false, true>(a, p, M, y, ldy, B, s);
-  return launch_pair_as<HD, G, W8, false>(a, p, M, y, ldy, B, s);
+  const bool eager = a.chunk_max > 128;  // more than half of a wave's four key tiles in use
+  if (!W8 && M >= XLDS_M16_FROM)
+    return eager ? launch_pair_as<HD, G, false, true, true>(a, p, M, y, ldy, B, s)
+                 : launch_pair_as<HD, G, false, true, false>(a, p, M, y, ldy, B, s);
+  return eager ? launch_pair_as<HD, G, W8, false, true>(a, p, M, y, ldy, B, s)
+               : launch_pair_as<HD, G, W8, false, false>(a, p, M, y, ldy, B, s);
 }
 
 // shared body of the two entry points; `fill` turns the caller's projection into a Proj
