@@ -115,17 +115,24 @@ __global__ __launch_bounds__(256) void k_add_rmsnorm(const u16* __restrict__ rin
   __syncthreads();
   ss = (red[0] + red[1]) + (red[2] + red[3]);
   const float inv = rsqrtf(ss / (float)dim + eps);
+  // (all results first, in registers of their own, then all stores: a store's data registers cannot be reused
+  // before the store has completed, and with one set of them the compiler waits for the previous store in front of
+  // every conversion)
+  uint4 on[NORM_MAXIT];
+#pragma unroll
+  for (int it = 0; it < NORM_MAXIT; ++it) {
+    if (it * 256 * 8 >= dim) break;
+    float g[8], o[8];
+    unpack8(qg[it], g);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = round_bf(r[it][j] * inv) * g[j];
+    on[it] = pack8(o);
+  }
 #pragma unroll
   for (int it = 0; it < NORM_MAXIT; ++it) {
     const int c = (tid + it * 256) * 8;
     if (it * 256 * 8 >= dim) break;
-    if (c < dim) {
-      float g[8], o[8];
-      unpack8(qg[it], g);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) o[j] = round_bf(r[it][j] * inv) * g[j];
-      st16(nout + base + c, pack8(o));
-    }
+    if (c < dim) st16(nout + base + c, on[it]);
   }
 }
 
@@ -207,22 +214,32 @@ __global__ __launch_bounds__(256) void k_ladder_norms(const u16* __restrict__ ri
   __syncthreads();
   const float inv1 = rsqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)dim + eps);
   const float inv2 = rsqrtf(((red[4] + red[5]) + (red[6] + red[7])) / (float)dim + eps);
+  // (all results first, in registers of their own, then all stores: a store's data registers cannot be reused
+  // before the store has completed, and with one set of them the compiler waits for the previous stores in front of
+  // every conversion)
+  uint4 o1[NORM_MAXIT], o2[NORM_MAXIT];
+#pragma unroll
+  for (int it = 0; it < NORM_MAXIT; ++it) {
+    if (it * 256 * 8 >= dim) break;
+    float r[8], g[8], o[8];
+    unpack8(qr[it], r);
+    unpack8(qg1[it], g);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = round_bf(r[j] * inv1) * g[j];
+    o1[it] = pack8(o);
+    unpack8(q2[it], r);
+    unpack8(qg2[it], g);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = round_bf(r[j] * inv2) * g[j];
+    o2[it] = pack8(o);
+  }
 #pragma unroll
   for (int it = 0; it < NORM_MAXIT; ++it) {
     const int c = (tid + it * 256) * 8;
     if (it * 256 * 8 >= dim) break;
     if (c < dim) {
-      float r[8], g[8], o[8];
-      unpack8(qr[it], r);
-      unpack8(qg1[it], g);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) o[j] = round_bf(r[j] * inv1) * g[j];
-      st16(n1 + base + c, pack8(o));
-      unpack8(q2[it], r);
-      unpack8(qg2[it], g);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) o[j] = round_bf(r[j] * inv2) * g[j];
-      st16(n2 + base + c, pack8(o));
+      st16(n1 + base + c, o1[it]);
+      st16(n2 + base + c, o2[it]);
     }
   }
 }
