@@ -47,7 +47,7 @@ static int launch_decode(const u16* q, int64_t ldq, const u16* kc, const u16* vc
   if (!lr_raise_lds_limit(reinterpret_cast<const void*>(&k_attn_decode_partial<HD, G>), lds, lds_raised)) return LR_E_LAUNCH;
   k_attn_decode_partial<HD, G><<<dim3(nsplit, Hkv, B), dim3(256), lds, s>>>(q, ldq, kc, vc, pos, o_part, ml_part, Hkv,
                                                                             Smax, nsplit, chunk_max);
-  k_attn_decode_combine<HD><<<dim3(Hq, B), dim3(HD), 0, s>>>(o_part, ml_part, y, ldy, Hq, nsplit);
+  launch_attn_combine<HD>(o_part, ml_part, y, ldy, Hq, B, nsplit, s);
   return lr_launch_status();
 }
 

@@ -288,3 +288,45 @@ __global__ __launch_bounds__(HD) void k_attn_decode_combine(const float* __restr
   }
   y[(int64_t)b * ldy + h * HD + d] = f_to_bf(L > 0.0f ? o / L : 0.0f);
 }
+
+// The same for up to 32 * NB <= 64 splits.  The merge is a chain of memory round trips and little else, so here all of
+// it is requested before anything is waited for: lane s of a wave asks for (max, sum) of split s, every lane for
+// its element of every partial result (no branch around a load: a split beyond the last reads the last one again
+// and gets weight zero).  The weights exp(m_s - max) are formed by the 64 lanes at once and handed round through
+// v_readlane: one round trip, where the loop above makes two per eight splits and a scalar load per split.  The
+// sums run over the splits in ascending order with the same operations: the results are the same bits.
+template <int HD, int NB>
+__global__ __launch_bounds__(HD) void k_attn_decode_combine_once(const float* __restrict__ o_part,
+                                                                 const float* __restrict__ ml_part,
+                                                                 u16* __restrict__ y, int64_t ldy, int Hq, int nsplit) {
+  constexpr int NS = 32 * NB;
+  const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x, lane = d & 63;
+  const float* ml = ml_part + ((int64_t)b * Hq + h) * nsplit * 2;
+  const float* op = o_part + ((int64_t)b * Hq + h) * nsplit * HD;
+  const int sl = lane < nsplit ? lane : nsplit - 1;
+  const float2 mlv = *reinterpret_cast<const float2*>(ml + 2 * sl);
+  float ov[NS];
+#pragma unroll
+  for (int j = 0; j < NS; ++j) ov[j] = op[(int64_t)(j < nsplit ? j : nsplit - 1) * HD + d];
+  const float M = wave_max(mlv.x);  // (lanes beyond the last split repeat it: the maximum is the same)
+  const float w_lane = (lane >= nsplit || mlv.x == -INFINITY) ? 0.0f : expf(mlv.x - M);  // an empty split: (-inf, 0, 0)
+  float L = 0.0f, o = 0.0f;
+#pragma unroll
+  for (int j = 0; j < NS; ++j) {
+    const float wgt = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(w_lane), j));
+    const float lj = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(mlv.y), j));
+    if (j < nsplit) {  // uniform (a sum must not see the -0.0 + 0.0 of a padded split)
+      L = fmaf(wgt, lj, L);
+      o = fmaf(wgt, ov[j], o);
+    }
+  }
+  y[(int64_t)b * ldy + h * HD + d] = f_to_bf(L > 0.0f ? o / L : 0.0f);
+}
+
+template <int HD>
+static inline void launch_attn_combine(const float* o_part, const float* ml_part, u16* y, int64_t ldy, int Hq, int B,
+                                       int nsplit, hipStream_t s) {
+  if (nsplit <= 32) k_attn_decode_combine_once<HD, 1><<<dim3(Hq, B), dim3(HD), 0, s>>>(o_part, ml_part, y, ldy, Hq, nsplit);
+  else if (nsplit <= 64) k_attn_decode_combine_once<HD, 2><<<dim3(Hq, B), dim3(HD), 0, s>>>(o_part, ml_part, y, ldy, Hq, nsplit);
+  else k_attn_decode_combine<HD><<<dim3(Hq, B), dim3(HD), 0, s>>>(o_part, ml_part, y, ldy, Hq, nsplit);
+}

@@ -60,7 +60,7 @@ static int launch_pair_as(const AttnItems& a, const Proj& p, int M, u16* y, int6
   static std::atomic<unsigned long long> lds_raised{0};
   if (!lr_raise_lds_limit(reinterpret_cast<const void*>(&k_attn_beside_band<HD, G, W8, XL, EAGER>), lds, lds_raised)) return LR_E_LAUNCH;
   k_attn_beside_band<HD, G, W8, XL, EAGER><<<dim3((unsigned)(a.n_items + p.nwg)), dim3(256), lds, s>>>(a, p, M);
-  k_attn_decode_combine<HD><<<dim3(Hq, B), dim3(HD), 0, s>>>(a.o_part, a.ml_part, y, ldy, Hq, a.nsplit);
+  launch_attn_combine<HD>(a.o_part, a.ml_part, y, ldy, Hq, B, a.nsplit, s);
   return lr_launch_status();
 }
 
