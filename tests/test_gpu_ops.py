@@ -560,6 +560,9 @@ def test_rope_kv_write_position_out_of_range_sets_the_error_word(hip):
     (1, 8, 1, 128, 2176, 2048), (1, 8, 1, 128, 2176, 0), (1, 8, 1, 128, 2176, 2175), (8, 8, 1, 128, 2176, 2100),
     (64, 8, 1, 128, 2176, 2111), (2, 32, 8, 128, 1280, 1033), (1, 32, 8, 64, 160, 131), (16, 16, 1, 128, 4160, 4100),
     (3, 4, 4, 64, 40, 17), (2, 8, 4, 128, 264, 200), (1, 16, 1, 128, 520, 519),
+    # a cache long enough for more than 64 key chunks (merged by the general loop, not in one round trip), and
+    # exactly 32 chunks
+    (1, 8, 1, 128, 20000, 19000), (16, 8, 1, 128, 2048, 2047),
 ])
 def test_attn_decode(hip, B, Hq, Hkv, hd, Smax, pos):
     q = rnd(B, Hq * hd, seed=21)
