@@ -61,6 +61,7 @@ extern "C" int lr_attn_decode(const void* q, int64_t ldq, const void* k_cache, c
   LR_REQUIRE_PTR(scratch);
   if (pos == nullptr) return LR_E_NULL;
   if (B <= 0 || Hq <= 0 || Hkv <= 0 || hd <= 0 || Smax <= 0 || Hq % Hkv) return LR_E_SHAPE;
+  if ((int64_t)Smax * hd * 2 >= 0x7fffffff) return LR_E_UNSUPPORTED;  // the rows of one (sequence, head) are addressed with 32-bit offsets
   if (ldq < (int64_t)Hq * hd || ldy < (int64_t)Hq * hd || B > 65535) return LR_E_SHAPE;
   if (ldq % 8 || ldy % 8) return LR_E_ALIGN;
   if (scratch_bytes < lr_attn_decode_scratch_bytes(B, Hq, hd, Smax)) return LR_E_SHAPE;
