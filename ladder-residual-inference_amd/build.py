@@ -16,6 +16,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "gpt_fast", "libladder_hip.so")
 PROF_LIB = os.path.join(HERE, "gpt_fast", "libladder_hip_prof.so")
+BAND_PROF_LIB = os.path.join(HERE, "gpt_fast", "libladder_hip_bandprof.so")
 HEADERS = [os.path.join(CSRC, h) for h in ("lr_common.h", "attn_decode_item.h", "stream_band.h")] + \
     [os.path.join(HERE, "..", "include", "ladder_hip.h")]
 # sources that compile another source under a switch
@@ -66,24 +67,35 @@ def build(force=False, verbose=True):
     return LIB
 
 
-def build_step_profile(force=False, verbose=True):
-    """A second library, gpt_fast/libladder_hip_prof.so, whose decode-step kernels (bf16 and e4m3 weights) record
-    wall-clock stamps per workgroup and phase (-DLR_STEP_PROFILE; read by step_phases.py).  The product library
-    carries none of it."""
+def _build_variant(lib, sources, define, suffix, force, verbose):
+    """`lib` = the product objects, with `sources` recompiled under `define`."""
     build(force=force, verbose=False)
-    step_sources = ("ladder_step.hip", "ladder_step_fp8.hip")
-    res = [_compile(os.path.join(CSRC, f), force, ("-DLR_STEP_PROFILE",), "_prof") for f in step_sources]
+    res = [_compile(os.path.join(CSRC, f), force, (define,), suffix) for f in sources]
     changed = any(c for _, c in res)
     objs = [os.path.join(OBJ, f.replace(".hip", ".o")) for f in sorted(os.listdir(CSRC))
-            if f.endswith(".hip") and f not in step_sources] + [o for o, _ in res]
-    if force or changed or _stale(PROF_LIB, objs):
-        r = subprocess.run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PROF_LIB] + objs,
+            if f.endswith(".hip") and f not in sources] + [o for o, _ in res]
+    if force or changed or _stale(lib, objs):
+        r = subprocess.run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + objs,
                            capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError("link failed:\n" + r.stderr)
     if verbose:
-        print(f"built {PROF_LIB}")
-    return PROF_LIB
+        print(f"built {lib}")
+    return lib
+
+
+def build_step_profile(force=False, verbose=True):
+    """A second library, gpt_fast/libladder_hip_prof.so, whose decode-step kernels (bf16 and e4m3 weights) record
+    wall-clock stamps per workgroup and phase (-DLR_STEP_PROFILE; read by step_phases.py).  The product library
+    carries none of it."""
+    return _build_variant(PROF_LIB, ("ladder_step.hip", "ladder_step_fp8.hip"), "-DLR_STEP_PROFILE", "_prof", force,
+                          verbose)
+
+
+def build_band_profile(force=False, verbose=True):
+    """gpt_fast/libladder_hip_bandprof.so: the weight-streaming band kernel of lr_linear_multi records wall-clock
+    stamps per wave (-DLR_BAND_PROFILE; read by band_phases.py).  The product library carries none of it."""
+    return _build_variant(BAND_PROF_LIB, ("stream_gemm.hip",), "-DLR_BAND_PROFILE", "_bandprof", force, verbose)
 
 
 if __name__ == "__main__":
@@ -91,7 +103,11 @@ if __name__ == "__main__":
     ap.add_argument("--force", action="store_true")
     ap.add_argument("--profile-step", action="store_true",
                     help="also build libladder_hip_prof.so (decode-step kernel with per-phase time stamps)")
+    ap.add_argument("--profile-bands", action="store_true",
+                    help="also build libladder_hip_bandprof.so (band kernel with per-wave time stamps)")
     args = ap.parse_args()
     build(force=args.force)
     if args.profile_step:
         build_step_profile(force=args.force)
+    if args.profile_bands:
+        build_band_profile(force=args.force)

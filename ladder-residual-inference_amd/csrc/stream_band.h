@@ -19,6 +19,19 @@ constexpr int XLDS_MIN_MT = 32;       // band heights that always read their inp
 constexpr int XLDS_M16_FROM = 9;      // input rows from which the 16-row band does too
 constexpr int AUX_WEIGHTS = 2;        // weights: non-temporal (every line is used exactly once)
 
+#ifdef LR_BAND_PROFILE
+// Profile builds only: when set (lr_band_profile, stream_gemm.hip), every wave of every band records 100 MHz
+// wall-clock stamps at six points -- 0 entry, 1 first requests made, 2 first chunk in LDS, 3 end of the K loop,
+// 4 partial sums exchanged (second barrier), 5 end -- at [(workgroup * NWV + wave) * 8 + point].
+static __device__ unsigned long long* g_band_prof;
+static __device__ unsigned g_band_prof_wgs;  // workgroups the buffer has room for; the others record nothing
+#define LR_BAND_STAMP(k)                                                                              \
+  if (g_band_prof && blockIdx.x < g_band_prof_wgs && lane == 0)                                       \
+    g_band_prof[((size_t)blockIdx.x * NWV + wave) * 8 + (k)] = wall_clock64();
+#else
+#define LR_BAND_STAMP(k)
+#endif
+
 struct Proj {
   const u16* x;
   const u16* w;
@@ -86,6 +99,7 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l16 = lane & 15, l4 = lane >> 4;
+  LR_BAND_STAMP(0)
   const int n_out = pair_off ? pair_off : N;         // output columns
   const int n0 = band * rpw;                          // first row (pair) of the band
   const int nrows = n_out - n0 < rpw ? n_out - n0 : rpw;
@@ -177,6 +191,7 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
     issue_w(s, wr[s]);
   }
   asm volatile("" ::: "memory");
+  LR_BAND_STAMP(1)
   for (int c0 = 0; c0 < nch; c0 += NS) {
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
@@ -199,6 +214,9 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
         }
       }
       asm volatile("" ::: "memory");
+#ifdef LR_BAND_PROFILE
+      if (ci == 0) { LR_BAND_STAMP(2) }
+#endif
       if constexpr (W8) {
         // 256 elements of K per chunk: the A fragments are taken in two halves to keep them at 32 registers
         issue_w(ci + NS, wr[s]);
@@ -253,6 +271,7 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
     }
   }
 
+  LR_BAND_STAMP(3)
   // ---- the waves' partial sums meet in LDS (accumulator element e of tile (u, mt): band row
   //      16 u + 4 (lane / 16) + e, input row 16 mt + lane % 16) and are added in wave order
   __syncthreads();
@@ -265,6 +284,7 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
 #pragma unroll
       for (int e = 0; e < 4; ++e) red[wave * WSTRIDE + ((u * MTILES + mt) * 4 + e) * 64 + lane] = acc[u][mt][e];
   __syncthreads();
+  LR_BAND_STAMP(4)
   const int rows_out = pair_off ? 16 : 16 * UNITS;
   if (rope_table != nullptr) {
     // The fused q/k/v projection of a decode step (one token per sequence: input row m is sequence m):
@@ -309,6 +329,7 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
       }
       *reinterpret_cast<u32*>(yg + (int64_t)m * ldy + n) = plain;
     }
+    LR_BAND_STAMP(5)
     return;
   }
   for (int o = tid; o < rows_out * MT; o += NWV * 64) {
@@ -335,6 +356,7 @@ __device__ __forceinline__ void stream_band(const Proj& p, const int M, const in
       yg[(int64_t)m * ldy + n0 + r] = f_to_bf(s0);
     }
   }
+  LR_BAND_STAMP(5)
 }
 
 // Rows per workgroup: the rows are spread evenly over whole rounds of the CUs, at most `cap` per

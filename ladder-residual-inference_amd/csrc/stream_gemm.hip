@@ -80,6 +80,22 @@ extern "C" int lr_linear_multi(const lr_projection_t* proj, int n_proj, int M, l
   return rc != LR_OK ? rc : lr_launch_status();
 }
 
+#ifdef LR_BAND_PROFILE
+// Profile builds only (not declared in the public header): following launches of this file's kernels record, per
+// wave, the six wall-clock stamps of stream_band.h into `device_buffer` (NULL switches it off).  Returns the
+// bytes the buffer must hold for the first `workgroups` workgroups of a launch (the others record nothing), or a
+// negative error code.
+extern "C" long long lr_band_profile(void* device_buffer, int workgroups) {
+  if (workgroups < 0) return LR_E_SHAPE;
+  unsigned long long* ptr = (unsigned long long*)device_buffer;
+  const unsigned wgs = (unsigned)workgroups;
+  if (hipMemcpyToSymbol(HIP_SYMBOL(g_band_prof), &ptr, sizeof(ptr)) != hipSuccess ||
+      hipMemcpyToSymbol(HIP_SYMBOL(g_band_prof_wgs), &wgs, sizeof(wgs)) != hipSuccess)
+    return LR_E_LAUNCH;
+  return (long long)workgroups * NWV * 8 * (long long)sizeof(unsigned long long);
+}
+#endif
+
 // lr_linear_fp8_multi (gemv_fp8.hip) for 3 to 16 input rows: the same bands with e4m3 weights.
 namespace lr_detail {
 int stream_fp8_multi(const lr_projection_fp8_t* proj, int n_proj, int M, lr_stream_t stream) {
