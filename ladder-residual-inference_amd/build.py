@@ -30,6 +30,11 @@ FLAGS = [
 ]
 
 
+# per-source additions: the prefill attention rescales its matrix-core accumulators with vector instructions; kept
+# in ordinary vector registers (not the accumulation registers) that costs no copies
+PER_SOURCE_FLAGS = {"attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+
+
 def _stale(target, deps):
     if not os.path.exists(target):
         return True
@@ -41,7 +46,7 @@ def _compile(src, force, extra=(), suffix=""):
     obj = os.path.join(OBJ, os.path.basename(src).replace(".hip", suffix + ".o"))
     if not force and not _stale(obj, [src] + HEADERS + INCLUDES.get(os.path.basename(src), [])):
         return obj, False
-    cmd = ["hipcc"] + FLAGS + list(extra) + ["-c", src, "-o", obj]
+    cmd = ["hipcc"] + FLAGS + PER_SOURCE_FLAGS.get(os.path.basename(src), []) + list(extra) + ["-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "is not a recognized feature for this target" not in l)
     if r.returncode != 0:

@@ -241,9 +241,23 @@ __global__ __launch_bounds__(64) void k_attn_prefill(const u16* __restrict__ q, 
 // (p = bf16(p) + bf16(p - bf16(p))), which keeps the fp32 softmax weights to ~2^-17: the result matches
 // the fp32 "math" attention of the eager reference (utils.py:247-258) to rounding of the final bf16.
 // A workgroup is 4 waves = NWH heads of one kv head x NWQ tiles of 32 queries sharing the K / V tiles.
-// e^x through the hardware exp2 (1 ulp in fp32: far below the bf16 rounding of the output); the
-// library expf costs ~15 VALU instructions, and this kernel is VALU-bound next to its MFMAs
-__device__ __forceinline__ float exp_fast(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+// e^x through the hardware exp2 (1 ulp in fp32: far below the bf16 rounding of the output), with the score scale
+// folded into its argument; the library expf costs ~15 VALU instructions, and this kernel is VALU-bound next to
+// its MFMAs
+// one v_max3_f32 (fmaxf written out makes the compiler canonicalise every operand first: an instruction each)
+__device__ __forceinline__ float max3_hw(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+__device__ __forceinline__ float exp2_hw(float x) { return __builtin_amdgcn_exp2f(x); }
+// two fp32 -> one dword of two bf16 (round to nearest even): a single v_cvt_pk_bf16_f32
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ u32 cvt_pk_bf2(float lo, float hi) {
+  return __builtin_bit_cast(u32, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
+}
+constexpr float PREFILL_TAU2 = 8.0f;  // log2 of the largest softmax weight before the reference point moves
 
 template <int HD, int NWH>
 __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const u16* __restrict__ q, int64_t ldq,
@@ -296,8 +310,17 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const u16* __restrict
   for (int d = 0; d < DT; ++d)
 #pragma unroll
     for (int v = 0; v < 16; ++v) o[d][v] = 0.0f;
-  float m = -INFINITY, l = 0.0f;  // l: this lane's half of the row sum
-  const float scale = rsqrtf((float)HD);
+  float m = -INFINITY, l = 0.0f;  // m: reference point in raw score units; l: this lane's half of the row sum
+  const float c2 = rsqrtf((float)HD) * 1.4426950408889634f;  // e^(x / sqrt(HD)) = 2^(x c2)
+  const float tau_raw = PREFILL_TAU2 / c2;
+  // the smallest position among the wave's queries (lanes without a query do not count)
+  int pmin = valid ? p : 0x7fffffff;
+#pragma unroll
+  for (int o_ = 32; o_ > 0; o_ >>= 1) {
+    const int t = __shfl_xor(pmin, o_, LR_WAVE);
+    pmin = t < pmin ? t : pmin;
+  }
+  pmin = __builtin_amdgcn_readfirstlane(pmin);
   const u16* kbase = kc + ((int64_t)b * Hkv + kvh) * Smax * HD;
   const u16* vbase = vc + ((int64_t)b * Hkv + kvh) * Smax * HD;
 
@@ -346,46 +369,44 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const u16* __restrict
       sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, ka), __builtin_bit_cast(bf16x8_t, qb[i]),
                                                      sacc, 0, 0, 0);
     }
-    // element v is key t0 + (v / 4) * 8 + half * 4 + v % 4 for query `col`
-    float tmax = -INFINITY;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int key = t0 + (v / 4) * 8 + half * 4 + (v % 4);
-      sacc[v] = key <= p ? sacc[v] * scale : -INFINITY;
-      tmax = fmaxf(tmax, sacc[v]);
-    }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, LR_WAVE));
-    const float mn = fmaxf(m, tmax);
-    float corr = 1.0f;
-    u32x4_t phi[2], plo[2];
-    if (mn != -INFINITY) {
-      corr = exp_fast(m - mn);  // m == -inf -> 0
-      l *= corr;
-      float pv[16];
+    // element v is key t0 + (v / 4) * 8 + half * 4 + v % 4 for query `col`; only a tile that reaches past the
+    // smallest position of the wave's queries has anything to mask
+    if (t0 + 31 > pmin) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        pv[v] = exp_fast(sacc[v] - mn);  // masked -> 0
-        l += pv[v];
+        const int key = t0 + (v / 4) * 8 + half * 4 + (v % 4);
+        sacc[v] = key <= p ? sacc[v] : -INFINITY;
       }
-#pragma unroll
-      for (int h2 = 0; h2 < 2; ++h2) {
-        u32 hi[4], lo[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float a0 = pv[8 * h2 + 2 * j], a1 = pv[8 * h2 + 2 * j + 1];
-          const float h0 = round_bf(a0), h1 = round_bf(a1);
-          hi[j] = pack_bf2(h0, h1);
-          lo[j] = pack_bf2(a0 - h0, a1 - h1);
-        }
-        phi[h2] = u32x4_t{hi[0], hi[1], hi[2], hi[3]};
-        plo[h2] = u32x4_t{lo[0], lo[1], lo[2], lo[3]};
-      }
-      m = mn;
-    } else {
-      phi[0] = phi[1] = plo[0] = plo[1] = u32x4_t{0u, 0u, 0u, 0u};
     }
+    float tmax = max3_hw(sacc[0], sacc[1], sacc[2]);
+#pragma unroll
+    for (int v = 3; v < 15; v += 2) tmax = max3_hw(tmax, sacc[v], sacc[v + 1]);
+    tmax = fmaxf(tmax, sacc[15]);
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, LR_WAVE));
+    // The reference point m of the exponentials follows the running maximum lazily: it moves only when a tile's
+    // maximum exceeds it by more than PREFILL_TAU2 / c2, so the weights stay below 2^PREFILL_TAU2 (harmless in fp32,
+    // and hi + lo keeps their relative precision) and the accumulators are rescaled on few tiles instead of on
+    // most (with 32 queries per wave, some running maximum moves in the majority of tiles).
+    const bool grow = tmax > m + tau_raw;  // m = -inf: any finite maximum
+    const float mn = grow ? tmax : m;
+    const float corr = grow ? exp2_hw((m - mn) * c2) : 1.0f;  // m = -inf -> 0
+    const float nmc = mn == -INFINITY ? 0.0f : -mn * c2;     // nothing seen yet: every score is -inf, weight 0
+    m = mn;
+    l *= corr;
+    u32x4_t phi[2], plo[2];
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float a0 = exp2_hw(fmaf(sacc[8 * h2 + 2 * j], c2, nmc));  // masked -> 0
+        const float a1 = exp2_hw(fmaf(sacc[8 * h2 + 2 * j + 1], c2, nmc));
+        l += a0 + a1;
+        const u32 hi = cvt_pk_bf2(a0, a1);
+        phi[h2][j] = hi;
+        plo[h2][j] = cvt_pk_bf2(a0 - __uint_as_float(hi << 16), a1 - __uint_as_float(hi & 0xffff0000u));
+      }
     // ---- O^T += V^T P^T ; k-step h2 covers keys 16 h2 + {0..3, 8..11} + 4 half, in the order of sacc
-    const bool rescale = __any(corr != 1.0f);  // the running maxima rarely move after the first tiles
+    const bool rescale = __any(grow);
 #pragma unroll
     for (int d = 0; d < DT; ++d) {
       if (rescale) {

@@ -682,6 +682,23 @@ def test_attn_prefill(hip, B, S, Hq, Hkv, hd, Smax, start):
     assert_close_ulp(y, want, max_frac=0.03, what="attn_prefill")
 
 
+@pytest.mark.parametrize("qscale", [4.0, 12.0])
+def test_attn_prefill_large_scores(hip, qscale):
+    """Scores with a standard deviation of 4 and 12: the running maximum of a query jumps by more than the kernel lets
+    its reference point lag, on tiles late in the history too, so accumulators are rescaled in mid-stream; and the
+    softmax is nearly one-hot at the larger scale."""
+    B, S, Hq, Hkv, hd, Smax = 2, 700, 8, 2, 128, 704
+    q = rnd(B, S, Hq * hd, seed=124, scale=qscale)
+    kc = rnd(B, Hkv, Smax, hd, seed=125)
+    vc = rnd(B, Hkv, Smax, hd, seed=126)
+    pos = torch.arange(S, dtype=torch.int32, device=DEV)
+    y = torch.empty(B, S, Hq * hd, dtype=BF, device=DEV)
+    hip.attn_prefill(q, kc, vc, pos, y, B, S, Hq, Hkv, hd)
+    mask = torch.arange(Smax, device=DEV).view(1, Smax) <= pos.view(S, 1)
+    want = O.sdpa_math(q.view(B, S, Hq, hd).transpose(1, 2), kc, vc, mask).transpose(1, 2).reshape(B, S, Hq * hd)
+    assert_close_ulp(y, want, max_frac=0.03, what="attn_prefill, large scores")
+
+
 # ------------------------------------------------------------------------------------ argmax
 
 def test_argmax_lowest_index_on_ties(hip):
