@@ -244,12 +244,11 @@ __global__ __launch_bounds__(64) void k_attn_prefill(const u16* __restrict__ q, 
 // e^x through the hardware exp2 (1 ulp in fp32: far below the bf16 rounding of the output), with the score scale
 // folded into its argument; the library expf costs ~15 VALU instructions, and this kernel is VALU-bound next to
 // its MFMAs
-// one v_max3_f32 (fmaxf written out makes the compiler canonicalise every operand first: an instruction each)
-__device__ __forceinline__ float max3_hw(float a, float b, float c) {
-  float r;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
-}
+// max(a, b) as the median of {a, b, +inf}: one instruction (fmaxf makes the compiler canonicalise both operands
+// first, an instruction each, when they come out of a matrix-core product).  Not for NaN operands.
+// (No inline assembler here: the compiler does not count the wait states between a matrix-core instruction and
+// an assembler statement that reads its result, and the statement then reads the registers too early.)
+__device__ __forceinline__ float max_med3(float a, float b) { return __builtin_amdgcn_fmed3f(a, b, INFINITY); }
 __device__ __forceinline__ float exp2_hw(float x) { return __builtin_amdgcn_exp2f(x); }
 // two fp32 -> one dword of two bf16 (round to nearest even): a single v_cvt_pk_bf16_f32
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
@@ -275,10 +274,22 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const u16* __restrict
   const int col = lane & 31, half = lane >> 5;
   const int G = Hq / Hkv;
   const int hgroups = G / NWH;                       // workgroups per kv head along heads
-  const int kvh = blockIdx.y / hgroups;
-  const int head = kvh * G + (blockIdx.y % hgroups) * NWH + (wave % NWH);
-  const int b = blockIdx.z;
-  const int s = (blockIdx.x * NWQ + wave / NWH) * 32 + col;  // this lane's query
+  // Which (query block, head group, sequence) this workgroup takes.  The grid is one-dimensional and workgroup i
+  // runs on XCD i % 8, each with an L2 of its own: XCD k takes the k-th eighth of the work in its logical order, so
+  // that the workgroups that share the K / V rows of one (sequence, kv head) -- the query blocks, neighbours in that
+  // order -- meet in one L2.  Inside, the query blocks go from the last (the longest history) to the first.
+  const int gx = (S + 32 * NWQ - 1) / (32 * NWQ), gy = Hq / NWH;
+  int wg;
+  {
+    const int n = gridDim.x, xcd = blockIdx.x % 8, idx = blockIdx.x / 8;
+    const int base = n / 8, rem = n % 8;
+    wg = xcd * base + (xcd < rem ? xcd : rem) + idx;
+  }
+  const int bx = gx - 1 - wg % gx, by = (wg / gx) % gy;
+  const int b = wg / (gx * gy);
+  const int kvh = by / hgroups;
+  const int head = kvh * G + (by % hgroups) * NWH + (wave % NWH);
+  const int s = (bx * NWQ + wave / NWH) * 32 + col;  // this lane's query
   const bool valid = s < S;
   int p = valid ? pos[s] : -1;
   p = p >= Smax ? Smax - 1 : p;
@@ -331,14 +342,18 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const u16* __restrict
   const int dch = tid % (HD / 8), kp = tid / (HD / 8);
   const bool stager = kp < 16;
   const int kps = kp ^ ((dch >> 2) * 4);
-  uint4 gk[2], gv[2];
+  // (buffer loads: a key beyond the needed range, or a thread without a staging slot, asks with an offset outside
+  // the resource and gets zeros -- no branch around a load)
+  u32x4_t gk[2], gv[2];
+  const __amdgpu_buffer_rsrc_t kres = __builtin_amdgcn_make_buffer_rsrc(const_cast<u16*>(kbase), 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t vres = __builtin_amdgcn_make_buffer_rsrc(const_cast<u16*>(vbase), 0, 0x7fffffff, 0x00020000);
+  const int stage_off = stager ? (2 * kp * HD + dch * 8) * 2 : (int)0x80000000;  // bytes, first key of the pair
   auto stage_load = [&](int t0) {
 #pragma unroll
     for (int e = 0; e < 2; ++e) {
-      const int key = t0 + 2 * kp + e;
-      const bool ok = stager && key < nkeys;
-      gk[e] = ok ? ld16(kbase + (int64_t)key * HD + dch * 8) : make_uint4(0, 0, 0, 0);
-      gv[e] = ok ? ld16(vbase + (int64_t)key * HD + dch * 8) : make_uint4(0, 0, 0, 0);
+      const int off = (stager && t0 + 2 * kp + e < nkeys) ? stage_off + (t0 + e) * HD * 2 : (int)0x80000000;
+      gk[e] = __builtin_amdgcn_raw_buffer_load_b128(kres, off, 0, 0);
+      gv[e] = __builtin_amdgcn_raw_buffer_load_b128(vres, off, 0, 0);
     }
   };
   stage_load(0);
@@ -348,8 +363,8 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const u16* __restrict
     // ---- 32 keys into LDS: K row-major, V transposed ([d][key], two keys per dword)
     if (stager) {
 #pragma unroll
-      for (int e = 0; e < 2; ++e) *reinterpret_cast<uint4*>(&ks[(2 * kp + e) * KROW + dch * 8]) = gk[e];
-      const u32 a4[4] = {gv[0].x, gv[0].y, gv[0].z, gv[0].w}, b4[4] = {gv[1].x, gv[1].y, gv[1].z, gv[1].w};
+      for (int e = 0; e < 2; ++e) *reinterpret_cast<u32x4_t*>(&ks[(2 * kp + e) * KROW + dch * 8]) = gk[e];
+      const u32 a4[4] = {gv[0][0], gv[0][1], gv[0][2], gv[0][3]}, b4[4] = {gv[1][0], gv[1][1], gv[1][2], gv[1][3]};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         vt32[(dch * 8 + 2 * j) * (VROW / 2) + kps] = (a4[j] & 0xffffu) | (b4[j] << 16);
@@ -378,10 +393,9 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const u16* __restrict
         sacc[v] = key <= p ? sacc[v] : -INFINITY;
       }
     }
-    float tmax = max3_hw(sacc[0], sacc[1], sacc[2]);
+    float tmax = max_med3(sacc[0], sacc[1]);
 #pragma unroll
-    for (int v = 3; v < 15; v += 2) tmax = max3_hw(tmax, sacc[v], sacc[v + 1]);
-    tmax = fmaxf(tmax, sacc[15]);
+    for (int v = 2; v < 16; ++v) tmax = max_med3(tmax, sacc[v]);
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, LR_WAVE));
     // The reference point m of the exponentials follows the running maximum lazily: it moves only when a tile's
     // maximum exceeds it by more than PREFILL_TAU2 / c2, so the weights stay below 2^PREFILL_TAU2 (harmless in fp32,
@@ -449,14 +463,14 @@ static int launch_prefill_mfma(const u16* q, int64_t ldq, const u16* kc, const u
                                int64_t ldy, int B, int S, int Hq, int Hkv, int Smax, hipStream_t s) {
   const int G = Hq / Hkv;
   if (G % 4 == 0) {
-    k_attn_prefill_mfma<HD, 4><<<dim3((S + 31) / 32, Hq / 4, B), dim3(256), 0, s>>>(q, ldq, kc, vc, pos, y, ldy, S, Hq,
-                                                                                  Hkv, Smax);
+    k_attn_prefill_mfma<HD, 4><<<dim3((unsigned)((int64_t)((S + 31) / 32) * (Hq / 4) * B)), dim3(256), 0, s>>>(
+        q, ldq, kc, vc, pos, y, ldy, S, Hq, Hkv, Smax);
   } else if (G % 2 == 0) {
-    k_attn_prefill_mfma<HD, 2><<<dim3((S + 63) / 64, Hq / 2, B), dim3(256), 0, s>>>(q, ldq, kc, vc, pos, y, ldy, S, Hq,
-                                                                                  Hkv, Smax);
+    k_attn_prefill_mfma<HD, 2><<<dim3((unsigned)((int64_t)((S + 63) / 64) * (Hq / 2) * B)), dim3(256), 0, s>>>(
+        q, ldq, kc, vc, pos, y, ldy, S, Hq, Hkv, Smax);
   } else {
-    k_attn_prefill_mfma<HD, 1><<<dim3((S + 127) / 128, Hq, B), dim3(256), 0, s>>>(q, ldq, kc, vc, pos, y, ldy, S, Hq,
-                                                                                Hkv, Smax);
+    k_attn_prefill_mfma<HD, 1><<<dim3((unsigned)((int64_t)((S + 127) / 128) * Hq * B)), dim3(256), 0, s>>>(
+        q, ldq, kc, vc, pos, y, ldy, S, Hq, Hkv, Smax);
   }
   return lr_launch_status();
 }
@@ -475,6 +489,10 @@ extern "C" int lr_attn_prefill(const void* q, int64_t ldq, const void* k_cache, 
   const dim3 grid((S + 63) / 64, Hq, B);
   hipStream_t s = (hipStream_t)stream;
   if (S >= 16 && Hq <= 65535 * 4) {  // matrix-core kernel; the lane-per-query kernel below serves short inputs
+    // (its staging addresses the rows of one (sequence, kv head) with 32-bit byte offsets)
+    if ((hd == 128 || hd == 64) && (int64_t)Smax * hd * 2 >= 0x7fffffff) return LR_E_UNSUPPORTED;
+    // (and its grid is one-dimensional, at most (S / 32) * Hq * B workgroups of 256 lanes: 2^32 lanes is the limit)
+    if ((hd == 128 || hd == 64) && (int64_t)((S + 31) / 32) * Hq * B >= (1 << 24)) return LR_E_UNSUPPORTED;
     if (hd == 128)
       return launch_prefill_mfma<128>((const u16*)q, ldq, (const u16*)k_cache, (const u16*)v_cache, pos, (u16*)y, ldy,
                                       B, S, Hq, Hkv, Smax, s);
