@@ -421,24 +421,33 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const u16* __restrict
       }
     // ---- O^T += V^T P^T ; k-step h2 covers keys 16 h2 + {0..3, 8..11} + 4 half, in the order of sacc
     const bool rescale = __any(grow);
+    if (rescale) {
 #pragma unroll
-    for (int d = 0; d < DT; ++d) {
-      if (rescale) {
+      for (int d = 0; d < DT; ++d)
 #pragma unroll
         for (int v = 0; v < 16; ++v) o[d][v] *= corr;
-      }
+    }
+    // (consecutive matrix instructions go to different accumulators: one that adds to the result of the instruction
+    // right before it has to wait for that result)
 #pragma unroll
-      for (int h2 = 0; h2 < 2; ++h2) {
-        // keys 16 h2 + 4 half + {0..3} and + 8 + {0..3}; rows of tile d were stored with pairs XOR 4 d
+    for (int h2 = 0; h2 < 2; ++h2) {
+      // keys 16 h2 + 4 half + {0..3} and + 8 + {0..3}; rows of tile d were stored with pairs XOR 4 d
+      u32x4_t va[DT];
+#pragma unroll
+      for (int d = 0; d < DT; ++d) {
         const u16* vr = &vt[(d * 32 + col) * VROW];
         const uint2 v0 = *reinterpret_cast<const uint2*>(vr + ((16 * h2 + 4 * half) ^ (8 * d)));
         const uint2 v1 = *reinterpret_cast<const uint2*>(vr + ((16 * h2 + 8 + 4 * half) ^ (8 * d)));
-        const u32x4_t va = {v0.x, v0.y, v1.x, v1.y};
-        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, va), __builtin_bit_cast(bf16x8_t, phi[h2]),
-                                                       o[d], 0, 0, 0);
-        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, va), __builtin_bit_cast(bf16x8_t, plo[h2]),
-                                                       o[d], 0, 0, 0);
+        va[d] = u32x4_t{v0.x, v0.y, v1.x, v1.y};
       }
+#pragma unroll
+      for (int d = 0; d < DT; ++d)
+        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, va[d]),
+                                                       __builtin_bit_cast(bf16x8_t, phi[h2]), o[d], 0, 0, 0);
+#pragma unroll
+      for (int d = 0; d < DT; ++d)
+        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, va[d]),
+                                                       __builtin_bit_cast(bf16x8_t, plo[h2]), o[d], 0, 0, 0);
     }
   }
   l += __shfl_xor(l, 32, LR_WAVE);
