@@ -137,6 +137,11 @@ __global__ __launch_bounds__(256) void k_gemm(const u16* __restrict__ x, int64_t
 // ---------------------------------------------------------------------------------------------
 constexpr int GM = 256, GN = 256;
 
+// KTAIL: K is not a multiple of the 64-element k-tile, so the last tile needs a per-lane range check.  Without it the
+// k position of a load is a scalar added by the load instruction itself and the row part of the address never
+// changes: no vector instruction per load (with the check: add, select and a 16-register offset update per tile,
+// ~60 vector instructions that the matrix instructions wait behind).
+template <bool KTAIL>
 __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int64_t ldx, const u16* __restrict__ w,
                                                   u16* __restrict__ y, int64_t ldy, int M, int N, int K, int tm,
                                                   int tn, int pair_off) {
@@ -192,9 +197,24 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
       woff[i] = n0 + r < N ? r * K * 2 : (int)0x80000000;
     }
   }
+  // k = first element of the k-tile (the same for all lanes); a tile beyond K is only ever requested, never used
+  // (the two tiles asked for past the end): without the per-lane check it is replaced by the last real tile
+  const int klast = ((K + BK - 1) / BK - 1) * BK;
+  if (!KTAIL) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (xoff[i] >= 0) xoff[i] += scol * 2;
+      if (woff[i] >= 0) woff[i] += scol * 2;
+    }
+  }
   auto fetch = [&](const __amdgpu_buffer_rsrc_t& res, int rowoff, int k) -> uint4 {
-    const int off = (k < K && rowoff >= 0) ? rowoff + k * 2 : (int)0x80000000;
-    const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(res, off, 0, 0);
+    u32x4_t v;
+    if (KTAIL) {
+      const int off = (k + scol < K && rowoff >= 0) ? rowoff + (k + scol) * 2 : (int)0x80000000;
+      v = __builtin_amdgcn_raw_buffer_load_b128(res, off, 0, 0);
+    } else {
+      v = __builtin_amdgcn_raw_buffer_load_b128(res, rowoff, (k < klast ? k : klast) * 2, 0);
+    }
     return make_uint4(v.x, v.y, v.z, v.w);
   };
   // Global -> LDS staging one tile ahead through ONE register set, in quarters: while tile kt is
@@ -205,8 +225,8 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
   const int nk = (K + BK - 1) / BK;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    xr[i] = fetch(xres, xoff[i], scol);
-    wr[i] = fetch(wres, woff[i], scol);
+    xr[i] = fetch(xres, xoff[i], 0);
+    wr[i] = fetch(wres, woff[i], 0);
   }
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -217,8 +237,8 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
   // loads in flight never depends on a branch and the waits can be exact)
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    xr[i] = fetch(xres, xoff[i], BK + scol);
-    wr[i] = fetch(wres, woff[i], BK + scol);
+    xr[i] = fetch(xres, xoff[i], BK);
+    wr[i] = fetch(wres, woff[i], BK);
   }
   __syncthreads();
 
@@ -266,8 +286,8 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
           else st16(&wn_[(srow0 + i * 32) * LDT + scol], wr[i]);
         } else if (ft >= 0 && ft < 4) {
           const int i = 2 * ks + (ft >> 1);
-          if ((ft & 1) == 0) xr[i] = fetch(xres, xoff[i], k2 + scol);
-          else wr[i] = fetch(wres, woff[i], k2 + scol);
+          if ((ft & 1) == 0) xr[i] = fetch(xres, xoff[i], k2);
+          else wr[i] = fetch(wres, woff[i], k2);
         }
         __builtin_amdgcn_sched_barrier(0);
         if (last && j == 3) {
@@ -347,11 +367,19 @@ static int launch_gemm_big(const void* x, int64_t ldx, const void* w, void* y, i
                            int pair_off, hipStream_t s) {
   constexpr size_t lds = (size_t)2 * (GM + GN) * LDT * sizeof(u16);
   static std::atomic<unsigned long long> lds_raised{0};
-  if (!lr_raise_lds_limit(reinterpret_cast<const void*>(&k_gemm_big), lds, lds_raised)) return LR_E_LAUNCH;
+  static std::atomic<unsigned long long> lds_raised_tail{0};
+  const bool ktail = K % BK != 0;
+  if (!(ktail ? lr_raise_lds_limit(reinterpret_cast<const void*>(&k_gemm_big<true>), lds, lds_raised_tail)
+              : lr_raise_lds_limit(reinterpret_cast<const void*>(&k_gemm_big<false>), lds, lds_raised)))
+    return LR_E_LAUNCH;
   const int gn = pair_off ? GN / 2 : GN;
   const int tm = (M + GM - 1) / GM, tn = (N + gn - 1) / gn;
-  k_gemm_big<<<dim3((unsigned)(tm * tn)), dim3(256), lds, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy, M, N, K,
-                                                              tm, tn, pair_off);
+  if (ktail)
+    k_gemm_big<true><<<dim3((unsigned)(tm * tn)), dim3(256), lds, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy, M,
+                                                                      N, K, tm, tn, pair_off);
+  else
+    k_gemm_big<false><<<dim3((unsigned)(tm * tn)), dim3(256), lds, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy,
+                                                                       M, N, K, tm, tn, pair_off);
   return lr_launch_status();
 }
 
