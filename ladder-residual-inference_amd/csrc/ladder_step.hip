@@ -118,7 +118,7 @@ struct LayerPtrs {
 
 struct StepParams {
   int D, L, Hkv, I, V, vocab, Smax, block_size, B, NA, nqkv;
-  int NAK, NAH;  // NA = NAK key ranges x NAH groups of kv heads: attention workgroup w takes range w % NAK of group w / NAK
+  int NAK, NAH;  // NA = NAK key ranges x NAH groups of (sequence, kv head) pairs: attention workgroup w takes range w % NAK of group w / NAK
   float eps;
   const u16 *tok_emb, *final_norm, *out_w, *rope;
   const LayerPtrs* layers;
@@ -1386,14 +1386,15 @@ __global__ __launch_bounds__(NT) void k_ladder_step(const StepParams p) {
       LayerPtrs lcache;  // only the cache pointers are used
       lcache.k_cache = const_cast<u16*>(ring_ptr(lring, t, LP_K_CACHE));
       lcache.v_cache = const_cast<u16*>(ring_ptr(lring, t, LP_V_CACHE));
-      const int hpg = p.Hkv / p.NAH, kvh0 = (w / p.NAK) * hpg;  // this workgroup's kv heads
-      for (int b = 0; b < p.B; ++b)
-        for (int kvh = kvh0; kvh < kvh0 + hpg; ++kvh) {
-          attention_load<HD>(p, lcache, b, kvh, k0, k1, pos, kv);
-          attention_compute<M, HD, G>(p, coh, lcache, b, kvh, k0, k1, pos, tag, LR_STAMP_PTR, kv,
-                                      reinterpret_cast<u32*>(qs), sc, sc_ld, ored, reinterpret_cast<u32*>(knew), vnew,
-                                      s_m, s_l);
-        }
+      // this workgroup's (sequence, kv head) pairs: pair b * Hkv + kvh, NAH groups of them
+      const int ppg = p.B * p.Hkv / p.NAH, pair0 = (w / p.NAK) * ppg;
+      for (int pr = pair0; pr < pair0 + ppg; ++pr) {
+        const int b = pr / p.Hkv, kvh = pr - b * p.Hkv;
+        attention_load<HD>(p, lcache, b, kvh, k0, k1, pos, kv);
+        attention_compute<M, HD, G>(p, coh, lcache, b, kvh, k0, k1, pos, tag, LR_STAMP_PTR, kv,
+                                    reinterpret_cast<u32*>(qs), sc, sc_ld, ored, reinterpret_cast<u32*>(knew), vnew,
+                                    s_m, s_l);
+      }
       coh.at(LR_STAMP_PTR, 29);
       attention_merge_slice<M, HD>(p, coh, Hq, tag, wbuf, w);
       prime(LR_JOB(JK_WO, LP_WO), opaque_tid() & 63, pipe);
@@ -1547,12 +1548,14 @@ static int pick_na(int Smax, int hd, int nwg, int want_na) {
 struct AttSplit {
   int nak, nah;
 };
-static AttSplit pick_split(const lr_ladder_model_t* md, int nwg) {
+static AttSplit pick_split(const lr_ladder_model_t* md, int nwg, int B = 1) {
   const int hd = md->head_dim, hkv = md->n_kv_head;
   AttSplit a;
   if (hkv == 1) {
     a.nak = pick_na(md->smax, hd, nwg, md->attention_workgroups);
-    a.nah = 1;
+    // two sequences: each gets key-range workgroups of its own (walked one after the other by the same workgroups,
+    // the attention takes 22.5 us per layer against 16.3 us of up/gate on the 70B shard)
+    a.nah = (B == 2 && 2 * a.nak <= nwg / 4) ? 2 : 1;
     return a;
   }
   const int cap = att_capacity(hd) < 256 ? att_capacity(hd) : 256;
@@ -1652,9 +1655,9 @@ static int validate(const lr_ladder_model_t* md, int B) {
   // loop): a workgroup without a row of wqkv, or a weight-streaming workgroup without a row pair of w1, would not
   // be part of that chain.  Such shapes (fewer q/k/v rows than CUs) are left to the per-op kernels.
   if ((md->n_head + 2 * md->n_kv_head) * md->head_dim < nwg) return LR_E_UNSUPPORTED;
-  const AttSplit as = pick_split(md, nwg);
+  const AttSplit as = pick_split(md, nwg, B);
   if (as.nak > NA_MAX || (md->smax + as.nak - 1) / as.nak > att_capacity(md->head_dim) || as.nak * as.nah >= nwg ||
-      md->n_kv_head % as.nah)
+      (B * md->n_kv_head) % as.nah)
     return LR_E_UNSUPPORTED;
   if (md->ffn < nwg - as.nak * as.nah) return LR_E_UNSUPPORTED;
   if (!md->tok_embeddings || !md->norm || !md->output || !md->freqs_cis || !md->layers_dev) return LR_E_NULL;
@@ -1775,7 +1778,7 @@ extern "C" int LR_STEP_ENTRY(const lr_ladder_model_t* md, int batch, const int32
   StepParams sp;
   sp.D = md->dim; sp.L = md->n_layer; sp.Hkv = md->n_kv_head; sp.I = md->ffn; sp.V = md->out_rows;
   sp.vocab = md->vocab; sp.Smax = md->smax; sp.block_size = md->block_size; sp.B = batch;
-  const AttSplit as = pick_split(md, nwg);
+  const AttSplit as = pick_split(md, nwg, batch);
   sp.NAK = as.nak; sp.NAH = as.nah; sp.NA = as.nak * as.nah;
   sp.nqkv = (md->n_head + 2 * md->n_kv_head) * md->head_dim;
   sp.eps = md->eps;
