@@ -1540,7 +1540,7 @@ static int pick_na(int Smax, int hd, int nwg, int want_na) {
   return na;
 }
 
-// How the attention workgroups are laid out: `nak` key ranges times `nah` groups of kv heads.  With one kv
+// How the attention workgroups are laid out: `nak` key ranges times `nah` groups of (sequence, kv head) pairs.  With one kv
 // head per rank (a TP shard) that is pick_na key ranges.  With several kv heads a workgroup that walked all of
 // them one after the other would keep the weight-streaming workgroups waiting (8B model: 62 us of attention
 // against 34 us of w1 per layer), so every kv head gets workgroups of its own and the key ranges become as long
@@ -1569,9 +1569,10 @@ static AttSplit pick_split(const lr_ladder_model_t* md, int nwg, int B = 1) {
   const float keys = (float)((md->smax + a.nak - 1) / a.nak);
   float best = 3.0e38f;
   a.nah = 1;
-  for (int nah = 1; nah <= hkv; ++nah) {
-    if (hkv % nah || a.nak * nah > nwg / 2) continue;
-    const float t_att = 7.0f + (float)(hkv / nah) * (2.5f + 0.04f * keys);
+  const int pairs = B * hkv;  // (sequence, kv head) pairs to go round
+  for (int nah = 1; nah <= pairs; ++nah) {
+    if (pairs % nah || a.nak * nah > nwg / 2) continue;
+    const float t_att = 7.0f + (float)(pairs / nah) * (2.5f + 0.04f * keys);
     const float t_w1 = 4.0f * (float)md->ffn * (float)md->dim / (float)(nwg - a.nak * nah) / 30.0e3f;
     const float t = t_att > t_w1 ? t_att : t_w1;
     if (t < best) { best = t; a.nah = nah; }
