@@ -256,7 +256,8 @@ size_t lr_attn_decode_scratch_bytes(int B, int Hq, int hd, int Smax);
  * the device, y [B, Hq*hd] (row stride ldy).  Only slots 0..pos are read; the reference reads
  * the whole cache under a mask (repeat_interleave + F.scaled_dot_product_attention,
  * utils.py:252-255, mask gpt_ladder_TP.py:254), which is the same function.  fp32 throughout,
- * one rounding of y.  scratch: lr_attn_decode_scratch_bytes(). */
+ * one rounding of y.  scratch: lr_attn_decode_scratch_bytes().  The rows of one (sequence, kv
+ * head) are addressed with 32-bit byte offsets: Smax * hd * 2 >= 2^31 - 1 is LR_E_UNSUPPORTED. */
 int lr_attn_decode(const void* q, int64_t ldq, const void* k_cache, const void* v_cache, const int32_t* pos, void* y,
                    int64_t ldy, int B, int Hq, int Hkv, int hd, int Smax, void* scratch, size_t scratch_bytes,
                    lr_stream_t stream);
@@ -279,7 +280,10 @@ int lr_attn_decode_static(const void* q, int64_t ldq, const void* k_cache, const
 /* Causal attention of S query tokens per sequence against the cache (prefill, S > 1):
  * query s of row b sits at position pos[s] and sees cache slots j <= pos[s].
  * q [B*S, Hq*hd] (row stride ldq), y [B*S, Hq*hd] (row stride ldy); the caches must already hold
- * this call's keys (lr_rope_kv_write).  Same maths and call sites as lr_attn_decode. */
+ * this call's keys (lr_rope_kv_write).  Same maths and call sites as lr_attn_decode.  From 16
+ * queries per sequence on (hd 64 or 128) the matrix-core kernel runs: Smax * hd * 2 >= 2^31 - 1 or
+ * more than 2^24 query blocks ((S / 32) * Hq * B) are LR_E_UNSUPPORTED.  Equal sequences give equal
+ * rows, bit for bit. */
 int lr_attn_prefill(const void* q, int64_t ldq, const void* k_cache, const void* v_cache, const int32_t* pos, void* y,
                     int64_t ldy, int B, int S, int Hq, int Hkv, int hd, int Smax, lr_stream_t stream);
 
