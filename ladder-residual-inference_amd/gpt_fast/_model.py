@@ -29,7 +29,7 @@ class Workspace:
         self.B, self.S, self.rows = B, S, rows
         self.x = e(rows, D)        # residual stream
         self.xn = e(rows, D)       # normed input of the current module
-        self.xn2 = e(rows, D) if S == 1 else None   # decode: the MLP's normed input while attention runs beside it
+        self.xn2 = e(rows, D)      # the MLP's normed input, formed together with the attention's (ladder schedule)
         self.a = e(rows, D)        # attention partial sum (pending in the ladder schedule)
         self.m = e(rows, D)        # MLP partial sum
         self.qkv = e(rows, fused_width)

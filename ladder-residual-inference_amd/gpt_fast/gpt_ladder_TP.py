@@ -230,6 +230,16 @@ class GPTLadder(GPTBase):
         if ws.S == 1 and cfg.ladder_layers is None:
             return self._run_layers_decode(ws, pos)
         pending_a = pending_m = None  # the reference starts from zero tensors; adding zero is the identity
+        if cfg.ladder_layers is None:
+            # all-ladder prefill: both residual updates and both norms of a block in one pass over the rows
+            # (lr_ladder_norms, as in decode: six tensor passes instead of the eight of two lr_add_rmsnorm)
+            for blk in self.layers:
+                _hip.ladder_norms(ws.x, pending_a, pending_m, blk.attention_norm.weight, blk.ffn_norm.weight, ws.x,
+                                  ws.xn, ws.xn2, eps)
+                self._attention(ws, blk, pos, blk.attention.wqkv, ws.a)
+                self._mlp(ws, blk, ws.m, ws.xn2)
+                pending_a, pending_m = ws.a, ws.m
+            return pending_a, pending_m
         for i, blk in enumerate(self.layers):
             if cfg.is_ladder_layer(i):
                 _hip.add_rmsnorm(ws.x, pending_a, None, blk.attention_norm.weight, ws.x, ws.xn, eps)
