@@ -147,6 +147,17 @@ typedef struct lr_projection {
 } lr_projection_t;
 int lr_linear_multi(const lr_projection_t* projections, int n_projections, int M, lr_stream_t stream);
 
+/* The fused q/k/v projection of a PREFILL, finished as lr_rope_kv_write would finish it: M = B * S input rows (S
+ * tokens per sequence, row b * S + s sits at position rope->pos[s], pos int32 [S] on the device),
+ * y[M, N] = x[M, K] w[N, K]^T with N = (n_head + 2 n_kv_head) * head_dim, then q rotated in y, rotated k and
+ * v stored at slot pos[s] of the caches, k and v left as projected in y (Attention.forward, utils.py:188-198, and
+ * KVCache.update, :50-59) -- bit for bit what lr_linear followed by lr_rope_kv_write (table_is_gathered = 0)
+ * leaves, in one launch of the prefill GEMM where that kernel applies (M >= 512 and enough tiles), in those two
+ * calls otherwise.  A position outside the cache or the table sets *rope->err = LR_DEV_POS_RANGE and leaves that
+ * row as projected.  ldy % 8 == 0. */
+int lr_linear_rope_kv(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int K, int S,
+                      const lr_rope_kv_t* rope, lr_stream_t stream);
+
 /* The MLP's first projection with the activation applied on the way out (utils.py:145-148):
  *     y[M, I] = bf16( bf16(silu(g)) * u ),  [u | g] = bf16(x w^T),  w [2 I, K] = [up; gate] rows, N = 2 I.
  * M <= 64: lr_linear_multi's LR_EPI_SWIGLU; M >= 512 on a large enough grid: the 256 x 256 tile

@@ -293,27 +293,6 @@ extern "C" int lr_swiglu(const void* h, int64_t ldh, void* out, int rows, int I,
 }
 
 // ------------------------------------------------------------------------------------ RoPE + KV write
-// 8 consecutive elements = 4 interleaved (even, odd) pairs; their (cos, sin) entries are the 8
-// consecutive bf16 at table[pos, d/2 .. d/2+3, :].  Products are rounded separately (no FMA
-// contraction) to reproduce the element-wise eager evaluation bit for bit.
-__device__ __forceinline__ uint4 rope8(const uint4& xv, const uint4& tv) {
-#pragma clang fp contract(off)
-  float x[8], t[8], o[8];
-  unpack8(xv, x);
-  unpack8(tv, t);
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const float c = t[2 * i], s = t[2 * i + 1];
-    const float a = x[2 * i] * c;
-    const float b = x[2 * i + 1] * s;
-    const float d = x[2 * i + 1] * c;
-    const float e = x[2 * i] * s;
-    o[2 * i] = a - b;
-    o[2 * i + 1] = d + e;
-  }
-  return pack8(o);
-}
-
 __global__ __launch_bounds__(256) void k_rope_kv_write(u16* qkv, int64_t ldqkv, const u16* __restrict__ table,
                                                        int table_is_gathered, const int32_t* __restrict__ pos,
                                                        u16* __restrict__ k_cache,

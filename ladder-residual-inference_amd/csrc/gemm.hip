@@ -141,10 +141,19 @@ constexpr int GM = 256, GN = 256;
 // k position of a load is a scalar added by the load instruction itself and the row part of the address never
 // changes: no vector instruction per load (with the check: add, select and a 16-register offset update per tile,
 // ~60 vector instructions that the matrix instructions wait behind).
-template <bool KTAIL>
+// ROPE: the projection is the fused q/k/v projection of a prefill (row b * S + s sits at position rpos[s]) and its
+// output pass does what k_rope_kv_write would do to the stored rows: q rotated in y, rotated k and plain v into the
+// caches, k and v left as projected in y; a position outside the cache or the table sets the error word and leaves
+// the plain row.
+struct GemmRope {
+  int S, Hq, Hkv, hd, Smax, block_size;
+};
+template <bool KTAIL, bool ROPE>
 __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int64_t ldx, const u16* __restrict__ w,
                                                   u16* __restrict__ y, int64_t ldy, int M, int N, int K, int tm,
-                                                  int tn, int pair_off) {
+                                                  int tn, int pair_off, const u16* __restrict__ rtable,
+                                                  const int32_t* __restrict__ rpos, u16* __restrict__ rk,
+                                                  u16* __restrict__ rv, int32_t* rerr, const GemmRope rp) {
   extern __shared__ __attribute__((aligned(16))) u16 gsm[];
   u16* xs = gsm;                      // [2][GM * LDT]
   u16* ws = gsm + 2 * GM * LDT;       // [2][GN * LDT]
@@ -341,11 +350,19 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
     const bool vec_ok = (ldy & 7) == 0;
     const int cl = (lane % LPR) * 8;
     const int ncol0 = n0 + wn * WN + cl;
-#pragma unroll 4
-    for (int r0 = 0; r0 < 128; r0 += RPI) {
-      const int ml = r0 + lane / LPR;
-      const int m = m0 + wm * 128 + ml;
-      const uint4 v = *reinterpret_cast<const uint4*>(&eb[ml * EP + cl]);
+    // ROPE: the lane's eight columns lie in one head of one section (head_dim % 8 == 0); its rows are RPI apart
+    int rb = 0, rs = 0, sect = 0, hh = 0, dd = 0;
+    if constexpr (ROPE && !P) {
+      const int mfirst = m0 + wm * 128 + lane / LPR;
+      rb = mfirst / rp.S;
+      rs = mfirst - rb * rp.S;
+      const int nq = rp.Hq * rp.hd, nkv = rp.Hkv * rp.hd;
+      sect = ncol0 < nq ? 0 : (ncol0 < nq + nkv ? 1 : 2);
+      const int cc = ncol0 - (sect == 0 ? 0 : (sect == 1 ? nq : nq + nkv));
+      hh = cc / rp.hd;
+      dd = cc - hh * rp.hd;
+    }
+    auto store_row = [&](int m, const uint4& v) {
       if (m < M) {
         if (vec_ok && ncol0 + 7 < N) {
           *reinterpret_cast<uint4*>(y + (int64_t)m * ldy + ncol0) = v;
@@ -356,31 +373,83 @@ __global__ __launch_bounds__(256) void k_gemm_big(const u16* __restrict__ x, int
             if (ncol0 + e < N) y[(int64_t)m * ldy + ncol0 + e] = (u16)(q[e >> 1] >> ((e & 1) * 16));
         }
       }
+    };
+    if constexpr (ROPE && !P) {
+      // Sixteen rows at a time: all their positions first, then all their table entries, then the arithmetic -- two
+      // memory round trips per sixteen rows (row by row the position and the table entry it selects are a chain of
+      // two dependent loads per row, and the output pass of a tile took three times as long).
+      constexpr int RB = 16;
+      for (int h0 = 0; h0 < 128 / RPI; h0 += RB) {
+        int ps[RB], bb[RB];
+#pragma unroll
+        for (int i = 0; i < RB; ++i) {
+          bb[i] = rb;
+          const int m = m0 + wm * 128 + (h0 + i) * RPI + lane / LPR;
+          ps[i] = (m < M && ncol0 < N) ? rpos[rs] : -1;  // (N % 8 == 0 and ldy % 8 == 0 here: the column group is whole)
+          rs += RPI;
+          while (rs >= rp.S) { rs -= rp.S; ++rb; }
+        }
+        uint4 tv[RB];
+        bool ok[RB];
+#pragma unroll
+        for (int i = 0; i < RB; ++i) {
+          ok[i] = ps[i] >= 0 && ps[i] < rp.Smax && ps[i] < rp.block_size;
+          tv[i] = (ok[i] && sect < 2) ? ld16(rtable + (int64_t)ps[i] * rp.hd + dd) : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < RB; ++i) {
+          const int ml = (h0 + i) * RPI + lane / LPR;
+          const int m = m0 + wm * 128 + ml;
+          uint4 v = *reinterpret_cast<const uint4*>(&eb[ml * EP + cl]);
+          if (ok[i]) {
+            const uint4 r = sect < 2 ? rope8(v, tv[i]) : v;
+            if (sect == 0) v = r;
+            else st16((sect == 1 ? rk : rv) + (((int64_t)bb[i] * rp.Hkv + hh) * rp.Smax + ps[i]) * rp.hd + dd, r);
+          } else if (m < M && ncol0 < N && rerr && cl == 0 && wn == 0) {
+            *rerr = LR_DEV_POS_RANGE;
+          }
+          store_row(m, v);
+        }
+      }
+      return;
+    }
+#pragma unroll 4
+    for (int r0 = 0; r0 < 128; r0 += RPI) {
+      const int ml = r0 + lane / LPR;
+      store_row(m0 + wm * 128 + ml, *reinterpret_cast<const uint4*>(&eb[ml * EP + cl]));
     }
   };
   if (pair_off) emit(std::true_type{});
   else emit(std::false_type{});
 }
 
-// pair_off != 0: N counts [up; gate] row pairs (see the kernel)
-static int launch_gemm_big(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
-                           int pair_off, hipStream_t s) {
+// pair_off != 0: N counts [up; gate] row pairs (see the kernel); rope != nullptr: the q/k/v projection of a prefill
+// of S tokens per sequence (pair_off == 0, ldy % 8 == 0)
+template <bool KTAIL, bool ROPE>
+static int launch_gemm_big_as(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
+                              int pair_off, const lr_rope_kv_t* rope, int S, hipStream_t s) {
   constexpr size_t lds = (size_t)2 * (GM + GN) * LDT * sizeof(u16);
   static std::atomic<unsigned long long> lds_raised{0};
-  static std::atomic<unsigned long long> lds_raised_tail{0};
-  const bool ktail = K % BK != 0;
-  if (!(ktail ? lr_raise_lds_limit(reinterpret_cast<const void*>(&k_gemm_big<true>), lds, lds_raised_tail)
-              : lr_raise_lds_limit(reinterpret_cast<const void*>(&k_gemm_big<false>), lds, lds_raised)))
-    return LR_E_LAUNCH;
+  if (!lr_raise_lds_limit(reinterpret_cast<const void*>(&k_gemm_big<KTAIL, ROPE>), lds, lds_raised)) return LR_E_LAUNCH;
   const int gn = pair_off ? GN / 2 : GN;
   const int tm = (M + GM - 1) / GM, tn = (N + gn - 1) / gn;
-  if (ktail)
-    k_gemm_big<true><<<dim3((unsigned)(tm * tn)), dim3(256), lds, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy, M,
-                                                                      N, K, tm, tn, pair_off);
-  else
-    k_gemm_big<false><<<dim3((unsigned)(tm * tn)), dim3(256), lds, s>>>((const u16*)x, ldx, (const u16*)w, (u16*)y, ldy,
-                                                                       M, N, K, tm, tn, pair_off);
+  GemmRope rp = {};
+  if (ROPE) rp = GemmRope{S, rope->n_head, rope->n_kv_head, rope->head_dim, rope->smax, rope->block_size};
+  k_gemm_big<KTAIL, ROPE><<<dim3((unsigned)(tm * tn)), dim3(256), lds, s>>>(
+      (const u16*)x, ldx, (const u16*)w, (u16*)y, ldy, M, N, K, tm, tn, pair_off, ROPE ? (const u16*)rope->table : nullptr,
+      ROPE ? rope->pos : nullptr, ROPE ? (u16*)rope->k_cache : nullptr, ROPE ? (u16*)rope->v_cache : nullptr,
+      ROPE ? rope->err : nullptr, rp);
   return lr_launch_status();
+}
+
+static int launch_gemm_big(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
+                           int pair_off, hipStream_t s, const lr_rope_kv_t* rope = nullptr, int S = 0) {
+  const bool ktail = K % BK != 0;
+  if (rope)
+    return ktail ? launch_gemm_big_as<true, true>(x, ldx, w, y, ldy, M, N, K, pair_off, rope, S, s)
+                 : launch_gemm_big_as<false, true>(x, ldx, w, y, ldy, M, N, K, pair_off, rope, S, s);
+  return ktail ? launch_gemm_big_as<true, false>(x, ldx, w, y, ldy, M, N, K, pair_off, nullptr, 0, s)
+               : launch_gemm_big_as<false, false>(x, ldx, w, y, ldy, M, N, K, pair_off, nullptr, 0, s);
 }
 
 extern "C" int lr_linear_tuned(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
@@ -416,6 +485,34 @@ extern "C" int lr_linear_tuned(const void* x, int64_t ldx, const void* w, void* 
 extern "C" int lr_linear(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int N, int K,
                          int act_swiglu, lr_stream_t stream) {
   return lr_linear_tuned(x, ldx, w, y, ldy, M, N, K, act_swiglu, 0, stream);
+}
+
+// The fused q/k/v projection of M = B * S rows (S tokens per sequence, row b * S + s at position pos[s]) finished as
+// lr_rope_kv_write would finish it.  One launch where the 256 x 256-tile GEMM applies; otherwise the two calls.
+extern "C" int lr_linear_rope_kv(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int M, int K, int S,
+                                 const lr_rope_kv_t* rope, lr_stream_t stream) {
+  LR_REQUIRE_PTR(x);
+  LR_REQUIRE_PTR(w);
+  LR_REQUIRE_PTR(y);
+  if (rope == nullptr || rope->pos == nullptr) return LR_E_NULL;
+  LR_REQUIRE_PTR(rope->table);
+  LR_REQUIRE_PTR(rope->k_cache);
+  LR_REQUIRE_PTR(rope->v_cache);
+  if (M <= 0 || K <= 0 || S <= 0 || M % S) return LR_E_SHAPE;
+  if (rope->n_head <= 0 || rope->n_kv_head <= 0 || rope->head_dim <= 0 || rope->smax <= 0 || rope->block_size <= 0)
+    return LR_E_SHAPE;
+  const int64_t n64 = (int64_t)(rope->n_head + 2 * rope->n_kv_head) * rope->head_dim;
+  if (n64 > 0x7fffffff || ldx < K || ldy < n64) return LR_E_SHAPE;
+  if (K % 8 || ldx % 8 || ldy % 8 || rope->head_dim % 8) return LR_E_ALIGN;
+  const int N = (int)n64;
+  hipStream_t s = (hipStream_t)stream;
+  if (M >= 512 && N >= 256 && ((M + GM - 1) / GM) * ((N + GN - 1) / GN) >= 192 && (int64_t)GM * ldx * 2 < 0x7fffffff &&
+      (int64_t)GN * K * 2 < 0x7fffffff)
+    return launch_gemm_big(x, ldx, w, y, ldy, M, N, K, 0, s, rope, S);
+  const int rc = lr_linear(x, ldx, w, y, ldy, M, N, K, 0, stream);
+  if (rc != LR_OK) return rc;
+  return lr_rope_kv_write(y, ldy, rope->table, 0, rope->pos, rope->k_cache, rope->v_cache, M / S, S, rope->n_head,
+                          rope->n_kv_head, rope->head_dim, rope->smax, rope->block_size, rope->err, stream);
 }
 
 // y[M, I] = bf16( bf16(silu(g)) * u ) for [u | g] = x w^T with w = [up; gate] rows (N = 2 I): the MLP's first

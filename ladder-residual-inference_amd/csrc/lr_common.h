@@ -65,6 +65,27 @@ __device__ __forceinline__ uint4 pack8(const float* f) {
   return v;
 }
 
+// RoPE on 8 consecutive elements = 4 interleaved (even, odd) pairs; their (cos, sin) entries are the 8
+// consecutive bf16 at table[pos, d/2 .. d/2+3, :].  Products are rounded separately (no FMA
+// contraction) to reproduce the element-wise eager evaluation bit for bit.
+__device__ __forceinline__ uint4 rope8(const uint4& xv, const uint4& tv) {
+#pragma clang fp contract(off)
+  float x[8], t[8], o[8];
+  unpack8(xv, x);
+  unpack8(tv, t);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float c = t[2 * i], s = t[2 * i + 1];
+    const float a = x[2 * i] * c;
+    const float b = x[2 * i + 1] * s;
+    const float d = x[2 * i + 1] * c;
+    const float e = x[2 * i] * s;
+    o[2 * i] = a - b;
+    o[2 * i + 1] = d + e;
+  }
+  return pack8(o);
+}
+
 // Reductions over the 64 lanes of a wave, every lane getting the result.  Call them with all lanes active.
 // The 16-lane rows are folded with DPP rotations (vector ALU, no LDS crossbar: a __shfl_xor is a ds_bpermute with
 // the latency of an LDS access, six of them in a row for one sum), the four row results meet through scalar registers.

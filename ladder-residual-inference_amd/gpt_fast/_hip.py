@@ -37,6 +37,8 @@ _PROTOS = {
                                  c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "lr_kv_update": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int,
                              c_int, c_int, c_int, c_void_p, c_void_p]),
+    "lr_linear_rope_kv": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p,
+                                  c_void_p]),
     "lr_attn_decode_scratch_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "lr_attn_decode": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int,
                                c_int, c_int, c_void_p, c_size_t, c_void_p]),
@@ -210,14 +212,28 @@ class _Projection(ctypes.Structure):   # lr_projection_t
 EPI_NONE, EPI_SWIGLU, EPI_ROPE_KV = 0, 1, 2
 
 
-def rope_kv_epilogue(table, pos, k_cache, v_cache, Hq, Hkv, hd):
-    """The descriptor an EPI_ROPE_KV projection of linear_multi carries (decode: one token per sequence)."""
-    assert pos.dtype == torch.int32 and pos.is_cuda and pos.numel() == 1
+def rope_kv_epilogue(table, pos, k_cache, v_cache, Hq, Hkv, hd, n_pos=1):
+    """The descriptor an EPI_ROPE_KV projection of linear_multi carries (decode: one token per sequence), or
+    linear_rope_kv (prefill: `n_pos` tokens per sequence)."""
+    assert pos.dtype == torch.int32 and pos.is_cuda and pos.numel() == n_pos
     assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape == v_cache.shape
     _, hkv_c, Smax, hd_c = k_cache.shape
     assert hkv_c == Hkv and hd_c == hd and table.is_contiguous() and table.shape[-2:] == (hd // 2, 2)
     return _RopeKv(_dev(table), pos.data_ptr(), _dev(k_cache), _dev(v_cache),
                    device_error_word(k_cache.device).data_ptr(), Hq, Hkv, hd, Smax, table.shape[0])
+
+
+def linear_rope_kv(x, w, out, table, pos, k_cache, v_cache, B, S, Hq, Hkv, hd):
+    """The fused q/k/v projection of B * S rows, rotated and cached on its way out (lr_linear_rope_kv): what
+    linear(x, w, out) followed by rope_kv_write(out, table, False, pos, ...) leaves."""
+    M, K, ldx = _rows_ld(x)
+    Mo, N, ldy = _rows_ld(out)
+    assert M == Mo == B * S and w.is_contiguous() and tuple(w.shape) == ((Hq + 2 * Hkv) * hd, K) and N == w.shape[0]
+    assert B <= k_cache.shape[0]
+    rope = rope_kv_epilogue(table, pos, k_cache, v_cache, Hq, Hkv, hd, n_pos=S)
+    _check(load().lr_linear_rope_kv(_dev(x), ldx, _dev(w), _dev(out), ldy, M, K, S, ctypes.byref(rope), _stream()),
+           "lr_linear_rope_kv")
+    return out
 
 
 def linear_multi(*projections):

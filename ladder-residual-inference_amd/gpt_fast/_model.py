@@ -192,6 +192,11 @@ class GPTBase(nn.Module):
         if wqkv is not None and bands and not roped:
             _hip.linear_multi((ws.xn, wqkv.weight, ws.qkv, _hip.rope_kv_epilogue(self.freqs_cis, pos, kc, vc, Hq, Hkv, hd)))
             roped = True
+        elif (wqkv is not None and S > 1 and not roped and not hasattr(wqkv, "scales")
+              and wqkv.weight.shape[0] == (Hq + 2 * Hkv) * hd):   # (not the parallel family's wider projection)
+            # prefill: the projection rotates q and caches rotated k and v on its way out (one launch of the GEMM)
+            _hip.linear_rope_kv(ws.xn, wqkv.weight, ws.qkv, self.freqs_cis, pos, kc, vc, B, S, Hq, Hkv, hd)
+            roped = True
         elif wqkv is not None:
             _hip.module_linear(ws.xn, wqkv, ws.qkv)
         if not roped:

@@ -369,6 +369,69 @@ def test_rope_kv_write_exact(hip, hd, Hq, Hkv, gathered):
     assert torch.equal(work[..., Hq * hd:], torch.cat([k, v], -1))   # k and v columns are left as they were
 
 
+@pytest.mark.parametrize("B,S,Hq,Hkv,hd,K,Smax,start", [
+    # the 256 x 256-tile GEMM with the rotation and the cache writes in its output pass: whole tiles; ragged rows,
+    # sequences that end inside a tile, K with a tail, positions that do not start at 0; then shapes below that
+    # kernel's threshold (the two-call fallback) and a decode-sized one
+    (4, 1024, 16, 4, 128, 1024, 1024, 0), (5, 1000, 32, 16, 64, 520, 1072, 37), (9, 300, 16, 4, 128, 256, 512, 100),
+    (2, 100, 8, 1, 128, 512, 136, 0), (3, 1, 8, 2, 64, 264, 16, 5),
+])
+def test_linear_rope_kv_equals_the_two_calls(hip, B, S, Hq, Hkv, hd, K, Smax, start):
+    """lr_linear_rope_kv against lr_linear followed by lr_rope_kv_write on the same buffers: the output rows and both
+    caches bit for bit; and the separate calls against the oracle (apply_rope, kv_update) as everywhere."""
+    N = (Hq + 2 * Hkv) * hd
+    x = rnd(B * S, K, seed=80)
+    w = rnd(N, K, seed=81, scale=0.05)
+    pos = torch.arange(start, start + S, dtype=torch.int32, device=DEV)
+    table = O.rope_table(start + S + 3, hd, 500000, BF).to(DEV)
+    want = torch.empty(B * S, N, dtype=BF, device=DEV)
+    hip.linear(x, w, want)
+    proj = want.clone()
+    kc_w = torch.zeros(B + 1, Hkv, Smax, hd, dtype=BF, device=DEV)
+    vc_w = torch.zeros_like(kc_w)
+    hip.rope_kv_write(want, table, False, pos, kc_w, vc_w, B, S, Hq, Hkv, hd)
+    fc = table[pos.long()]
+    q, k, v = proj.view(B, S, N).split([Hq * hd, Hkv * hd, Hkv * hd], dim=-1)
+    assert torch.equal(want.view(B, S, N)[..., : Hq * hd].reshape(B, S, Hq, hd), O.apply_rope(q.reshape(B, S, Hq, hd), fc))
+    kc_o, vc_o = torch.zeros_like(kc_w), torch.zeros_like(kc_w)
+    O.kv_update(kc_o, vc_o, pos.long(), O.apply_rope(k.reshape(B, S, Hkv, hd), fc).transpose(1, 2),
+                v.reshape(B, S, Hkv, hd).transpose(1, 2))
+    assert torch.equal(kc_w, kc_o) and torch.equal(vc_w, vc_o)
+
+    got = torch.full((B * S, N), 7.0, dtype=BF, device=DEV)
+    kc, vc = torch.zeros_like(kc_w), torch.zeros_like(kc_w)
+    hip.linear_rope_kv(x, w, got, table, pos, kc, vc, B, S, Hq, Hkv, hd)
+    assert torch.equal(got, want)
+    assert torch.equal(kc, kc_w) and torch.equal(vc, vc_w)
+    hip.raise_on_device_error(got.device)
+
+
+def test_linear_rope_kv_position_out_of_range(hip):
+    """A position beyond the cache: that row stays as projected, nothing of it reaches the caches, the device error
+    word is set (as lr_rope_kv_write does); the other rows are finished as usual."""
+    B, S, Hq, Hkv, hd, K, Smax = 4, 1024, 16, 4, 128, 512, 1024
+    N = (Hq + 2 * Hkv) * hd
+    x, w = rnd(B * S, K, seed=82), rnd(N, K, seed=83, scale=0.05)
+    pos = torch.arange(S, dtype=torch.int32, device=DEV)
+    pos[700] = Smax + 5
+    table = O.rope_table(2048, hd, 500000, BF).to(DEV)
+    want = torch.empty(B * S, N, dtype=BF, device=DEV)
+    hip.linear(x, w, want)
+    kc_w = torch.zeros(B, Hkv, Smax, hd, dtype=BF, device=DEV)
+    vc_w = torch.zeros_like(kc_w)
+    hip.device_error_word(want.device).zero_()
+    hip.rope_kv_write(want, table, False, pos, kc_w, vc_w, B, S, Hq, Hkv, hd)
+    assert int(hip.device_error_word(want.device).item()) != 0
+    hip.device_error_word(want.device).zero_()
+    got = torch.empty_like(want)
+    kc, vc = torch.zeros_like(kc_w), torch.zeros_like(kc_w)
+    hip.linear_rope_kv(x, w, got, table, pos, kc, vc, B, S, Hq, Hkv, hd)
+    torch.cuda.synchronize()
+    assert int(hip.device_error_word(want.device).item()) != 0
+    hip.device_error_word(want.device).zero_()
+    assert torch.equal(got, want) and torch.equal(kc, kc_w) and torch.equal(vc, vc_w)
+
+
 @pytest.mark.parametrize("hd,H", [(128, 1), (64, 8), (128, 8)])
 @pytest.mark.parametrize("layout", ["bhsd", "bshd"])
 def test_kv_cache_update_module_method(hd, H, layout):
