@@ -89,6 +89,21 @@ def test_validation_precedes_any_device_work(lib):
     assert beside(64, ptr, 17) == -4                                # the 16-row band only
     assert beside(64, ptr, 4, epi=2) == -4                          # a projection that writes the cache
     assert beside(64, ptr, 4, scratch_bytes=16) == E_SHAPE
+    # the prefill's q/k/v projection with the rotation and the cache writes in its output pass
+    from gpt_fast._hip import _RopeKv
+    rope = _RopeKv(64, 128, 192, 256, None, 8, 1, 128, 64, 64)          # N = (8 + 2) * 128 = 1280
+
+    def fused(x=64, ldx=64, ldy=1280, M=8, K=64, S=4, r=rope):
+        return lib.lr_linear_rope_kv(x, ldx, 128, 256, ldy, M, K, S, None if r is None else ctypes.byref(r), None)
+
+    assert fused(x=None) == E_NULL
+    assert fused(r=None) == E_NULL
+    assert fused(M=9) == E_SHAPE                                        # whole sequences of S tokens
+    assert fused(ldy=1272) == E_SHAPE                                   # ldy < N
+    assert fused(ldy=1284) == E_ALIGN
+    assert fused(K=60, ldx=64) == E_ALIGN
+    assert fused(r=_RopeKv(64, None, 192, 256, None, 8, 1, 128, 64, 64)) == E_NULL      # no positions
+    assert fused(r=_RopeKv(64, 128, 192, 256, None, 8, 1, 124, 64, 64), ldy=1240) == E_ALIGN   # head_dim % 8
     from gpt_fast._hip import _ProjectionFp8
     one8 = (_ProjectionFp8 * 1)(_ProjectionFp8(64, 16, 128, 192, 256, 8, 8, 16, 0))
     ptr8 = ctypes.cast(one8, ctypes.c_void_p)
