@@ -252,7 +252,7 @@ def test_linear_multi_rope_kv_epilogue_reports_a_position_outside_the_cache(hip)
 
 
 @pytest.mark.parametrize("M,D,I", [(5, 264, 56), (64, 1024, 520), (100, 520, 136), (512, 4096, 14336 // 4), (700, 328, 1000),
-                                   (2048, 1024, 3584)])
+                                   (2048, 1024, 3584), (2300, 520, 3000), (2300, 512, 3000)])
 def test_linear_swiglu_out_equals_projection_then_swiglu(hip, M, D, I):
     """The first MLP projection with the activation in its epilogue -- the streaming kernel's row pairs (M <= 64), the
     256 x 256 tile GEMM on tiles of 128 pairs (M >= 512, ragged edges included), the two-step fallback in between --
@@ -308,7 +308,12 @@ def test_linear_gemv_is_deterministic(hip):
                                    # 256 x 256 tiles (M >= 512): whole tiles, ragged edges in M, N and K, the
                                    # XCD-aware tile order (M / 256 a multiple of 32) and the plain one
                                    (512, 256, 64), (700, 500, 328), (1024, 6144, 4096), (8192, 512, 136),
-                                   (8192 + 3, 257, 72)])
+                                   (8192 + 3, 257, 72),
+                                   # enough 256 x 256 tiles for the large-tile kernel (192 and more): whole tiles
+                                   # in the plain and in the XCD-aware order, ragged edges in M and N with K a
+                                   # multiple of the k-tile (scalar k offsets) and with a K tail (per-lane checks)
+                                   (4096, 3072, 1024), (8192, 1536, 512), (5000, 3000, 512), (5000, 3000, 328),
+                                   (6144, 2048, 64)])
 def test_linear_gemm(hip, M, N, K):
     x = rnd(M, K, seed=14)
     w = rnd(N, K, seed=15, scale=0.02)
