@@ -29,8 +29,8 @@ Prints ONE JSON line.  `value` = decoded tokens per second (whole job = the one 
                threads used (the process's CPU share: OMP_NUM_THREADS when set, else every core),
                `host_cpus` = os.cpu_count().
 Measured in the same run and reported as extra keys (not the headline; --no-extras skips them):
-`batched`     : the same rank shard at batch 8 and 64, the 8B model at batch 1 (one-kernel step) and 16 (prompt
-               1024) and the 405B rank shard at batch 16 (context 4096) -- per-op kernels unless noted,
+`batched`     : the same rank shard at batch 2 (one-kernel step), 4, 8 and 64, the 8B model at batch 1 (one-kernel
+               step) and 16 (prompt 1024) and the 405B rank shard at batch 16 (context 4096) -- per-op kernels unless noted,
                hipGraph replay: ms per step, tok/s, algorithmic GB/s and its fraction of 8 TB/s; `traffic` = HBM
                bytes per step from counter runs where one was made.
 `fp8`         : the same shard with weight-only e4m3 projections at batch 1 (the one-kernel step on e4m3 weights)
@@ -122,8 +122,9 @@ def decode_run(bm, model, prompt, B, T, K, W):
     return ms, first, dg
 
 
-def extra_batched(bm, model, prompt, T, batches=(4, 8, 64), K=32, W=5):
-    """The headline shard at the other batch sizes of the benchmark set (per-op kernels)."""
+def extra_batched(bm, model, prompt, T, batches=(2, 4, 8, 64), K=32, W=5):
+    """The headline shard at other batch sizes (2: the one-kernel step; from 3 on the per-op kernels; 4, 8 and 64 are
+    those of the benchmark set)."""
     cfg = model.config
     out = []
     for B in batches:
